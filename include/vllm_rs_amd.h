@@ -446,6 +446,9 @@ typedef struct vra_engine_config {
                                      reference defaults to 0.2); 0 = no swap space, preempted sequences wait or are dropped */
   int32_t swap_cooling_ms;        /* scheduler.rs:49 SWAP_COOLING_PERIOD; 0 = 5000, negative = none */
   int32_t min_tokens_left_for_swap; /* scheduler.rs:50; 0 = 1000, negative = 0 */
+  /* appended: slots for the per-sequence state of models whose layers carry one from token to token (linear-attention matrices, short
+   * convolutions, the previous token).  0 = one per sequence the scheduler may batch; fewer make sequences wait for a slot. */
+  int32_t num_state_slots;
 } vra_engine_config;
 
 /* Pure-host helpers (no GPU needed; also exported by libvra_host.so for CPU tests) */

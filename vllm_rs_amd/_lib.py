@@ -38,7 +38,7 @@ class EngineConfig(C.Structure):
         ("kv_fraction", c_f32), ("prefill_chunk", c_i32), ("enable_prefix_cache", c_i32),
         ("prefix_cache_fraction", c_f32), ("use_graph", c_i32), ("tp_rank", c_i32), ("tp_world_size", c_i32),
         ("device", c_i32), ("seed", c_u64), ("fp8_kvcache", c_i32), ("cpu_mem_fold", c_f32),
-        ("swap_cooling_ms", c_i32), ("min_tokens_left_for_swap", c_i32),
+        ("swap_cooling_ms", c_i32), ("min_tokens_left_for_swap", c_i32), ("num_state_slots", c_i32),
     ]
 
 

@@ -145,7 +145,70 @@ def parse_gaperax(cfg_json, dtype=None):
                 rms_norm_eps=float(norm.get("eps", 1e-6)), rope_theta=10000.0, dtype=dt, quant_method=None, spec="\n".join(lines) + "\n")
 
 
-STACK_ARCHS = {"Ditilix": parse_ditilix, "Gaperax": parse_gaperax}
+def parse_zifetar(cfg_json, dtype=None):
+    """Zifetar config.json -> cfg dict with arch "stack": sandwich-norm blocks (an RMS norm before and after every sub-block, weights stored
+    around zero), an embedding with a hashed token-pair table and a norm of its own, per layer one of three mixers that carry a state per
+    sequence (gated delta rule, retention, softmax attention inside blocks of positions beside a gated linear attention) and a mixture of
+    experts whose router takes a softmax over the chosen logits.  Every size and constant comes from the config; the ranks of the low-rank
+    projections come from the tensors' shapes ("rank_a" / "rank_g" of a mixer only size synthetic weights)."""
+    td = dtype or cfg_json.get("torch_dtype", "bfloat16")
+    dt = {"bfloat16": BF16, "bf16": BF16, "float32": F32, "f32": F32, BF16: BF16, F32: F32}.get(td)
+    if dt is None:
+        raise ValueError(f"dtype {td!r}: a layer stack runs in bfloat16 or float32")
+    norm = cfg_json.get("norm") or {}
+    em = cfg_json.get("embedding") or {}
+    bg = em.get("bigram") or {}
+    width, vocab, layers = int(cfg_json["width"]), int(cfg_json["vocab"]), cfg_json["layers"]
+    head = "stack width=%d vocab=%d eps=%s block=sandwich norm=rms pos=none norm_offset=1.0 embed_scale=%s embed_norm=1" % (
+        width, vocab, _num(norm.get("eps", 1e-6)), _num(em.get("scale", 1.0)))
+    if bg:
+        head += " pair_buckets=%d pair_mul_prev=%d pair_mul_cur=%d" % (int(bg["buckets"]), int(bg["mul_prev"]), int(bg["mul_cur"]))
+    lines = [head]
+    heads = kv_heads = dim = 1
+
+    def rot_fields(mx):
+        rot = mx.get("rot") or {}
+        f = dict(rot_dims=int(rot.get("dims", 0)), rot_base=_num(rot.get("base", 10000.0)))
+        sc = rot.get("scaling")
+        if sc:
+            f.update(rs_factor=_num(sc["factor"]), rs_low=_num(sc["low"]), rs_high=_num(sc["high"]), rs_original=_num(sc["original"]))
+        return f
+
+    for i, layer in enumerate(layers):
+        mx, kind = layer["mixer"], layer.get("type")
+        if kind == "channel_delta":
+            f = dict(mixer="delta", heads=int(mx["heads"]), kv_heads=int(mx.get("kv_heads", mx["heads"])), dim=int(mx["dim"]),
+                     vdim=int(mx.get("vdim", mx["dim"])), conv=int(mx.get("conv", 1)), rank_a=int(mx.get("rank_a", 16)), rank_g=int(mx.get("rank_g", 16)))
+        elif kind == "retention":
+            f = dict(mixer="retention", heads=int(mx["heads"]), dim=int(mx["dim"]), vdim=int(mx.get("vdim", mx["dim"])),
+                     decay=",".join(_num(d) for d in mx["decay"]))
+            f.update(rot_fields(mx))
+        elif kind == "parallel":
+            le, ri = mx["left"], mx["right"]
+            f = dict(mixer="parallel", heads=int(le["heads"]), kv_heads=int(le.get("kv_heads", le["heads"])), dim=int(le["dim"]),
+                     vdim=int(le.get("vdim", le["dim"])), scale=_num(le["scale"]) if le.get("scale") is not None else _num(int(le["dim"]) ** -0.5),
+                     chunk=int((le.get("mask") or {}).get("size", 0)), qk_norm=1, bias=1,
+                     r_heads=int(ri["heads"]), r_dim=int(ri["dim"]), r_vdim=int(ri.get("vdim", ri["dim"])), tau=_num(ri["tau"]),
+                     rank_a=int(ri.get("rank_a", 16)), left_scale=_num(mx.get("left_scale", 1.0)), right_scale=_num(mx.get("right_scale", 1.0)))
+            f.update(rot_fields(le))
+        else:
+            raise ValueError(f"layer {i}: mixer type {kind!r} is not part of this design")
+        mlp = layer.get("mlp")
+        if not mlp:
+            f.update(mlp="none")
+        elif mlp["kind"] == "moe":
+            f.update(mlp="moe", ff=int(mlp["expert"]["ff"]), experts=int(mlp["router"]["experts"]), top=int(mlp["router"].get("top", 1)),
+                     router="softmax", act="silu")
+        else:
+            raise ValueError(f"layer {i}: feed-forward kind {mlp['kind']!r} is not part of this design")
+        lines.append("layer " + " ".join(f"{k}={v}" for k, v in f.items()))
+        heads, kv_heads, dim = max(heads, f["heads"]), max(kv_heads, f.get("kv_heads", f["heads"])), max(dim, f["dim"], f["vdim"])
+    return dict(arch="stack", design="Zifetar", hidden_size=width, vocab_size=vocab, num_layers=len(layers), num_heads=heads, num_kv_heads=kv_heads,
+                head_dim=dim, intermediate_size=0, max_position_embeddings=int(cfg_json.get("max_position_embeddings", 1 << 20)),
+                rms_norm_eps=float(norm.get("eps", 1e-6)), rope_theta=10000.0, dtype=dt, quant_method=None, spec="\n".join(lines) + "\n")
+
+
+STACK_ARCHS = {"Ditilix": parse_ditilix, "Gaperax": parse_gaperax, "Zifetar": parse_zifetar}
 
 
 def parse_config(cfg_json, dtype=None):

@@ -3,6 +3,7 @@
 #include <math.h>
 
 #include "common.cuh"
+#include "stack_launch.h"
 
 namespace {
 
@@ -30,6 +31,24 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 __device__ __forceinline__ float sigmoidf_(float z) { return 1.f / (1.f + expf(-z)); }
+__device__ __forceinline__ float block_sum_256(float v, float* red) {
+  v = wave_sum(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+// cos / sin of p * (hi + lo), times mag: the product p * hi is split exactly (fma), the small part enters to first order
+__device__ __forceinline__ void rot_cos_sin(const StkRotary& r, int i, float p, float* c, float* s) {
+  const float fh = r.freq_hi[i], fl = r.freq_lo ? r.freq_lo[i] : 0.f;
+  const float ah = p * fh;
+  const float al = fmaf(p, fh, -ah) + p * fl;
+  const float c0 = cosf(ah), s0 = sinf(ah);
+  *c = (c0 - s0 * al) * r.mag;
+  *s = (s0 + c0 * al) * r.mag;
+}
+
 template <typename F>
 void launch_checked(const char* what, F f) {
   f();

@@ -30,7 +30,7 @@ struct StkGemmArgs {
   const int* out_row = nullptr;
   int epi = 0;
   float limit = 0.f, act_alpha = 1.702f;
-  int act = 0;                  // the gated pair of epi 1: 0 the clamped form above, 1  gelu_tanh(g) * u
+  int act = 0;                  // the gated pair of epi 1: 0 the clamped form above, 1  gelu_tanh(g) * u, 2  silu(g) * u
   const float* bias = nullptr;  // f32 [N], added after alpha (plain epilogue)
   // batched form (no row groups): product z of `batch` reads a + z * a_batch_stride, w + z * w_batch_stride and writes out + z * out_batch_stride
   // (element counts; a column offset per head turns one launch into a product per head)
@@ -103,6 +103,8 @@ struct StkAttnArgs {
   const float* sink = nullptr;  // f32 [H]: the softmax denominator also holds exp(sink[h]) — a term without key or value, counted once
   int k_ld = 0, v_ld = 0;       // elements between the rows of kc / vc (0: G * dim / G * vdim).  A latent cache keeps one row [c | rotated
                                 // part] per token: keys are the whole row, values its first columns (vc = kc, v_ld = k_ld)
+  int chunk = 0;                // > 0: key j is visible only if it lies in the query's own block of `chunk` positions,
+                                // floor(j / chunk) = floor(p_i / chunk); blocks count from position 0 of the sequence
 };
 void vra_stack_attention(const StkAttnArgs& a, int dtype, int64_t stream);
 
@@ -186,3 +188,144 @@ struct StkSigAttnArgs {
   int max_len = 0;
 };
 void vra_stack_sigmoid_attention(const StkSigAttnArgs& a, int dtype, int64_t stream);
+
+// ---------------------------------------------------------------------------------------------------------------------------------------
+// Operators of sandwich-norm blocks with recurrent mixers (stack_recurrent.hip).  A sequence's recurrent state lives in the slot
+// state_slots[b] names (-1: a padded lane, nothing is read or written); a sequence whose first token of the step stands at position 0
+// starts from zeros, whatever the slot holds.  cu_q null: one token per sequence.
+
+// x[t] = N(embed[id_t] * scale + table[row_t]; norm_w),  row_t = (prev_t * mul_prev + id_t * mul_cur) mod buckets, and row `buckets` (the
+// table's last) for a sequence's first token; prev_t is the token before t: the row before it in the step, or prev_tokens[b] for the first
+// row of sequence b (the engine keeps every sequence's tokens).  N(v; w) = v / sqrt(mean(v^2) + eps) * w; norm_w null: no norm.
+struct StkEmbedPairArgs {
+  const uint32_t* ids = nullptr;
+  const int64_t* positions = nullptr;
+  const uint32_t* cu_q = nullptr;
+  const uint32_t* prev_tokens = nullptr;  // [B]
+  const void* embed = nullptr;            // [V, W]
+  const void* table = nullptr;            // [buckets + 1, W]; null: no pair term
+  int buckets = 0;
+  int64_t mul_prev = 0, mul_cur = 0;
+  float scale = 1.f;
+  const float* norm_w = nullptr;
+  float eps = 1e-6f;
+  float* x = nullptr;
+  int T = 0, B = 0, W = 0, V = 0;
+};
+void vra_stack_embed_pair(const StkEmbedPairArgs& a, int dtype, int64_t stream);
+
+// The seam between two sub-blocks of a sandwich-norm stack, one launch:
+//   s = c1 * sum_{j < n1} pw[t * n1 + j] * p1[(t * n1 + j), :]  +  c2 * p2[t, :]      (pw null: weights 1; p2 null: no second part)
+//   x[t] += N(s; post_w)                                                              (post_w null: nothing is added)
+//   h[t]  = N(x[t]; pre_w)  in dtype                                                  (pre_w null: no h)
+// and, with router_w ([n_router, W] in dtype): z = router_w . h + router_bias on the unrounded h, the `top` largest (ties: the lower
+// index) -> pair_expert / pair_weight [T, top], weights = softmax over the chosen logits.  All f32.
+struct StkSandwichArgs {
+  float* x = nullptr;
+  const float* p1 = nullptr;
+  int n1 = 1;
+  const float* pw = nullptr;
+  float c1 = 1.f;
+  const float* p2 = nullptr;
+  float c2 = 1.f;
+  const float* post_w = nullptr;
+  const float* pre_w = nullptr;
+  void* h = nullptr;
+  float eps = 1e-6f;
+  int T = 0, W = 0;
+  const void* router_w = nullptr;
+  const float* router_bias = nullptr;
+  int n_router = 0, top = 0;
+  int* pair_expert = nullptr;
+  float* pair_weight = nullptr;
+};
+void vra_stack_sandwich_norm(const StkSandwichArgs& a, int dtype, int64_t stream);
+
+// Heads of one token from the f32 row of a joint projection: per head an optional RMS norm over `dim` (weight [dim] shared by the heads),
+// rotary on the first 2 * rot.pairs dimensions in the rotate-half layout (dimension i pairs with i + rot.pairs), a scale.
+// q heads -> q_out [T, q_ld]; k heads -> k_out: rows by token (slots null) or the paged cache's rows by slot; v -> v_out likewise (null:
+// not written).  out_f32: outputs are f32 instead of dtype.
+struct StkHeadPrepArgs {
+  const float* raw = nullptr;
+  int ld = 0, q_off = 0, k_off = 0, v_off = 0;
+  int Hq = 0, Hk = 0, dim = 0, nv = 0;
+  const float* qn_w = nullptr;
+  const float* kn_w = nullptr;
+  float eps = 1e-6f;
+  StkRotary rot;
+  float q_scale = 1.f, k_scale = 1.f;
+  const int64_t* positions = nullptr;
+  void* q_out = nullptr;
+  int q_ld = 0;
+  void* k_out = nullptr;
+  int k_ld = 0;
+  void* v_out = nullptr;
+  int v_ld = 0;
+  const int64_t* slots = nullptr;
+  int out_f32 = 0;
+  int T = 0;
+};
+void vra_stack_head_prep(const StkHeadPrepArgs& a, int dtype, int64_t stream);
+
+// Inputs of a gated delta rule from the f32 rows  raw = [q (G * dim) | k (G * dim) | v (H * vdim) | b (H)]  and  raw2 = [a (H * dim) | ..]:
+// q, k, v pass a causal convolution over time per channel (conv_w [C, taps], last column = the current token; the taps - 1 inputs before a
+// step's first row come from conv_state [slots, taps - 1, C], zeros for a sequence that starts) and silu; q and k heads become unit
+// vectors (x / sqrt(sum x^2 + 1e-6)), q times q_scale  -> qkv_out [T, C] f32;  beta = sigmoid(b) -> beta_out [T, H];
+// decay = exp(-rate[h] * softplus(a + dt_bias)) -> decay_out [T, H * dim].  vra_stack_conv_state_update then moves the state on.
+struct StkDeltaPrepArgs {
+  const float* raw = nullptr;
+  int ld = 0;
+  const float* raw2 = nullptr;
+  int ld2 = 0;
+  const float* conv_w = nullptr;
+  int taps = 1;
+  float* conv_state = nullptr;
+  const float* rate = nullptr;     // [H]
+  const float* dt_bias = nullptr;  // [H * dim]
+  float q_scale = 1.f;
+  float* qkv_out = nullptr;
+  float* beta_out = nullptr;
+  float* decay_out = nullptr;
+  const int64_t* positions = nullptr;
+  const uint32_t* cu_q = nullptr;
+  const int32_t* state_slots = nullptr;
+  int T = 0, B = 0, H = 0, G = 0, dim = 0, vdim = 0;
+};
+void vra_stack_delta_prep(const StkDeltaPrepArgs& a, int64_t stream);
+void vra_stack_conv_state_update(const StkDeltaPrepArgs& a, int64_t stream);
+
+// out = exp(-softplus(-z) * inv_tau) = sigmoid(z)^(1 / tau), element by element (f32 [T, n] with row strides)
+void vra_stack_sigmoid_pow(const float* z, int ldz, float* out, int ldo, int T, int n, float inv_tau, int64_t stream);
+
+// Linear recurrence over a sequence's tokens with a matrix state S [dim, vdim] per head (f32, kept as its transpose [slots, H, vdim, dim]):
+//   S <- diag(d_t) S   (d_t: decay [T, ldd], head h at column h * dim; or head_decay[h] for every row)
+//   u = v_t (beta null)   or   u = beta_t (v_t - S^T k_t)  (delta rule)
+//   S <- S + k_t u^T ;  o_t = S^T (q_scale q_t)
+// q / k head of value head h = h / qk_rep.  Tokens run one after the other in one fixed order of operations, so a step's cut leaves no trace.
+struct StkScanArgs {
+  const float* q = nullptr;
+  int ldq = 0;
+  const float* k = nullptr;
+  int ldk = 0;
+  const float* v = nullptr;
+  int ldv = 0;
+  const float* decay = nullptr;
+  int ldd = 0;
+  const float* head_decay = nullptr;
+  const float* beta = nullptr;
+  int ldb = 0;
+  float q_scale = 1.f;
+  float* state = nullptr;
+  const int32_t* state_slots = nullptr;
+  const int64_t* positions = nullptr;
+  const uint32_t* cu_q = nullptr;
+  float* out = nullptr;
+  int ldo = 0;
+  int B = 0, H = 0, qk_rep = 1, dim = 0, vdim = 0;
+};
+void vra_stack_linear_scan(const StkScanArgs& a, int64_t stream);
+
+// out[t, h * vdim + c] = o[t, h, c] / sqrt(mean_c(o^2) + eps) * w[c] * act(gate[t, h * vdim + c])   (w null: 1; gate null: no gate;
+// gate_act 1: silu, 2: sigmoid);  o f32 [T, H * vdim], out in dtype
+void vra_stack_head_norm_gate(const float* o, const float* w, const float* gate, int gate_ld, int gate_act, float eps, void* out, int T, int H, int vdim,
+                              int dtype, int64_t stream);

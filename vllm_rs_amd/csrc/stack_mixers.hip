@@ -12,24 +12,6 @@
 
 namespace {
 
-__device__ __forceinline__ float block_sum_256(float v, float* red) {
-  v = wave_sum(v);
-  __syncthreads();
-  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
-  __syncthreads();
-  return (red[0] + red[1]) + (red[2] + red[3]);
-}
-
-// cos / sin of p * (hi + lo), times mag: the product p * hi is split exactly (fma), the small part enters to first order
-__device__ __forceinline__ void rot_cos_sin(const StkRotary& r, int i, float p, float* c, float* s) {
-  const float fh = r.freq_hi[i], fl = r.freq_lo ? r.freq_lo[i] : 0.f;
-  const float ah = p * fh;
-  const float al = fmaf(p, fh, -ah) + p * fl;
-  const float c0 = cosf(ah), s0 = sinf(ah);
-  *c = (c0 - s0 * al) * r.mag;
-  *s = (s0 + c0 * al) * r.mag;
-}
-
 // ------------------------------------------------------------------------------------------------ Dynamic Tanh (+ residual sum)
 template <typename T>
 __global__ __launch_bounds__(256) void stk_dyt_kernel(float* x, const float* add, const float* w, const float* b, float alpha, T* h, int W, int64_t n) {

@@ -13,9 +13,10 @@
 namespace {
 
 __device__ __forceinline__ float gelu_tanh_(float z) { return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z))); }
-// act 0: min(g, L) * sigmoid(act_alpha * min(g, L)) * (clamp(u, +-L) + 1);  act 1: gelu_tanh(g) * u
+// act 0: min(g, L) * sigmoid(act_alpha * min(g, L)) * (clamp(u, +-L) + 1);  act 1: gelu_tanh(g) * u;  act 2: silu(g) * u
 __device__ __forceinline__ float gated_pair(float g, float u, float limit, float act_alpha, int act = 0) {
   if (act == 1) return gelu_tanh_(g) * u;
+  if (act == 2) return g * sigmoidf_(g) * u;
   if (limit > 0.f) {
     g = fminf(g, limit);
     u = fminf(fmaxf(u, -limit), limit);
@@ -531,14 +532,17 @@ __global__ __launch_bounds__(256) void stk_attn_prefill_kernel(StkAttnArgs a) {
     if (r < nq) v = El<T>::ld(q + (size_t)(t0 + r) * a.ldq + h * dim + d) * q_temperature(a.positions[t0 + r], a.temp_coef, a.temp_every);
     qs[i] = v;
   }
-  int64_t pq[4];
-  int64_t pmax = -1;
+  int64_t pq[4], plo[4];
+  int64_t pmax = -1, lo_min = INT64_MAX;
+  auto block_start = [&](int64_t p) { return a.chunk > 0 ? p / a.chunk * a.chunk : (int64_t)0; };  // first key a query at p may see
   for (int i = 0; i < 4; i++) {
     const int r = wave * 4 + i;
     pq[i] = r < nq ? a.positions[t0 + r] : -1;
+    plo[i] = pq[i] >= 0 ? block_start(pq[i]) : 0;
   }
-  for (int r = 0; r < nq; r++) pmax = max(pmax, a.positions[t0 + r]);
+  for (int r = 0; r < nq; r++) pmax = max(pmax, a.positions[t0 + r]), lo_min = min(lo_min, block_start(a.positions[t0 + r]));
   const int n_keys = (int)min((int64_t)a.context_lens[b], pmax + 1);
+  const int kt_begin = (int)(lo_min / KT) * KT;  // (tiles stay aligned to absolute positions)
   float m[4], l[4], acc[4][4];
   for (int i = 0; i < 4; i++) {
     m[i] = -INFINITY, l[i] = 0.f;
@@ -549,7 +553,7 @@ __global__ __launch_bounds__(256) void stk_attn_prefill_kernel(StkAttnArgs a) {
   const T* vc = (const T*)a.vc;
   const uint32_t* bt = a.block_tables + (size_t)b * a.max_blocks;
   const int kdim = a.k_ld ? a.k_ld : a.G * dim, vd_all = a.v_ld ? a.v_ld : a.G * vdim;
-  for (int kt0 = 0; kt0 < n_keys; kt0 += KT) {
+  for (int kt0 = kt_begin; kt0 < n_keys; kt0 += KT) {
     __syncthreads();
     for (int i = tid; i < KT * dim; i += 256) {
       const int j = i / dim, d = i % dim, key = kt0 + j;
@@ -573,7 +577,7 @@ __global__ __launch_bounds__(256) void stk_attn_prefill_kernel(StkAttnArgs a) {
     for (int i = 0; i < 4; i++) {
       const int r = wave * 4 + i;
       float s = -INFINITY;
-      if (lane < KT && pq[i] >= 0 && kt0 + lane <= pq[i] && kt0 + lane < n_keys) {
+      if (lane < KT && pq[i] >= 0 && kt0 + lane <= pq[i] && kt0 + lane >= plo[i] && kt0 + lane < n_keys) {
         float d0 = 0.f;
         for (int d = 0; d < dim; d++) d0 = fmaf(qs[r * dim + d], ks[lane * kld + d], d0);
         s = cap_score(d0 * a.scale, a.softcap);
@@ -648,10 +652,16 @@ __global__ __launch_bounds__(256) void stk_attn_prefill_mfma_kernel(StkAttnArgs 
   // keys this workgroup needs: up to the largest position of its rows
   int64_t pmax = pq;
   for (int o = 32; o > 0; o >>= 1) pmax = max(pmax, (int64_t)__shfl_xor((long long)pmax, o, 64));
-  __shared__ long long wmax[4];
-  if (lane == 0) wmax[wave] = pmax;
+  // block mask: this row sees the keys from key_lo on; the workgroup's tiles start at the tile of its smallest key_lo
+  const int64_t key_lo = a.chunk > 0 && pq >= 0 ? pq / a.chunk * a.chunk : 0;
+  int64_t lmin = pq >= 0 ? key_lo : INT64_MAX;
+  for (int o = 32; o > 0; o >>= 1) lmin = min(lmin, (int64_t)__shfl_xor((long long)lmin, o, 64));
+  __shared__ long long wmax[4], wmin[4];
+  if (lane == 0) wmax[wave] = pmax, wmin[wave] = lmin;
   __syncthreads();
   const int64_t gmax = max(max(wmax[0], wmax[1]), max(wmax[2], wmax[3]));
+  const int64_t gmin = min(min(wmin[0], wmin[1]), min(wmin[2], wmin[3]));
+  const int kt_begin = gmin == INT64_MAX ? 0 : (int)(gmin / 32) * 32;
   const int n_keys = (int)min((int64_t)a.context_lens[b], gmax + 1);
   const int n_keys_wave = (int)min((int64_t)n_keys, pmax + 1);
   const uint16_t* kc = (const uint16_t*)a.kc;
@@ -703,9 +713,9 @@ __global__ __launch_bounds__(256) void stk_attn_prefill_mfma_kernel(StkAttnArgs 
       }
     }
   };
-  request_tile(0, page_slot(0));
-  int64_t slot_next = page_slot(KT);
-  for (int kt0 = 0; kt0 < n_keys; kt0 += KT) {
+  request_tile(kt_begin, page_slot(kt_begin));
+  int64_t slot_next = page_slot(kt_begin + KT);
+  for (int kt0 = kt_begin; kt0 < n_keys; kt0 += KT) {
     u32x4 kfc[2][DC], vgc[NV][2];
     for (int u = 0; u < 2; u++)
       for (int c = 0; c < DC; c++) kfc[u][c] = kfn[u][c];
@@ -750,7 +760,7 @@ __global__ __launch_bounds__(256) void stk_attn_prefill_mfma_kernel(StkAttnArgs 
           const float y = fminf(fmaxf(x * two_inv_cap, -30.f), 30.f);
           x = a.softcap - two_cap * __builtin_amdgcn_rcpf(1.f + __expf(y));
         }
-        x = key < key_end ? x : -INFINITY;
+        x = key < key_end && key >= key_lo ? x : -INFINITY;
         sv[u * 4 + j] = x;
         tmax = fmaxf(tmax, x);
       }
@@ -856,13 +866,16 @@ __global__ __launch_bounds__(64 * STK_DW) void stk_attn_decode_kernel(StkAttnArg
   while (oc * 8 < vdim) oc <<= 1;
   const int co = lane & (oc - 1), kg = lane / oc, kpar = 64 / oc;
   float vacc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  for (int kt0 = wave * 64; kt0 < n_keys; kt0 += STK_DW * 64) {
+  // block mask: the keys from key_lo on; tiles stay aligned to absolute positions (the first one may begin below key_lo: those keys
+  // count with weight 0)
+  const int key_lo = a.chunk > 0 ? (int)(p / a.chunk * a.chunk) : 0;
+  for (int kt0 = key_lo / 64 * 64 + wave * 64; kt0 < n_keys; kt0 += STK_DW * 64) {
     const int key = kt0 + lane;
     float s = -INFINITY;
     if (key < n_keys) {
       const int64_t slot = (int64_t)bt[key / a.BS] * a.BS + key % a.BS;
       ss[wave * 64 + lane] = (int)slot;
-      s = cap_score(stk_dot_row<T>(qs, kc + slot * kdim + g * dim, dim) * a.scale, a.softcap);
+      if (key >= key_lo) s = cap_score(stk_dot_row<T>(qs, kc + slot * kdim + g * dim, dim) * a.scale, a.softcap);
     }
     const float mn = fmaxf(m, wave_max(s));  // (the tile's first key exists: mn is finite)
     const float pj = s > -INFINITY ? expf(s - mn) : 0.f;

@@ -1,0 +1,422 @@
+// stack_recurrent.hip — operators of sandwich-norm layer stacks whose mixers carry a state from token to token (host/stack_model.cpp; each is
+// specified in stack_launch.h), gfx950: the embedding with a hashed token-pair table, the seam between two sub-blocks (norm of a sub-block's
+// output, residual sum, norm of the next one's input, router), per-head norm / rotary / cache rows, the inputs of a gated delta rule
+// (short convolutions with their state, unit vectors, step sizes and decays), the linear recurrence itself and its output norm and gate.
+//
+// Everything here is f32 except what is stored for a matrix product (h, q, cache rows, the gated output): norms, routers, angles, decays and
+// their logarithms, the recurrent state and all that enters it.  Tokens of a sequence pass the recurrence one after the other in one fixed
+// order of operations, and a sequence's state sits in its slot between steps, so a token's result does not depend on how its prompt was cut,
+// on the rest of the batch or on the slot.
+#include <algorithm>
+
+#include "stack_common.cuh"
+#include "stack_launch.h"
+
+namespace {
+
+__device__ __forceinline__ float softplusf_(float z) { return fmaxf(z, 0.f) + log1pf(expf(-fabsf(z))); }
+__device__ __forceinline__ float siluf_(float z) { return z / (1.f + expf(-z)); }
+
+// sequence of row t in a step whose rows are cut by cu_q [B + 1] (cu_q null: one row per sequence)
+__device__ __forceinline__ int seq_of_row(const uint32_t* cu_q, int B, int t) {
+  if (!cu_q) return t;
+  int lo = 0, hi = B - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if ((int)cu_q[mid] <= t) lo = mid;
+    else hi = mid - 1;
+  }
+  return lo;
+}
+
+// ------------------------------------------------------------------------------------------------ embedding + token-pair table + norm
+template <typename T>
+__global__ __launch_bounds__(256) void stk_embed_pair_kernel(StkEmbedPairArgs a) {
+  extern __shared__ float lds[];
+  __shared__ float red[4];
+  float* xs = lds;
+  const int t = blockIdx.x, W = a.W, tid = threadIdx.x;
+  uint32_t id = a.ids[t];
+  if (id >= (uint32_t)a.V) id = 0;
+  const T* e = (const T*)a.embed + (size_t)id * W;
+  const T* pr = nullptr;
+  if (a.table) {
+    const int b = seq_of_row(a.cu_q, a.B, t);
+    const int t0 = a.cu_q ? (int)a.cu_q[b] : t;
+    int64_t row = a.buckets;
+    if (a.positions[t] > 0) {
+      const uint32_t prev = t > t0 ? a.ids[t - 1] : a.prev_tokens[b];
+      row = ((int64_t)prev * a.mul_prev + (int64_t)id * a.mul_cur) % (int64_t)a.buckets;
+      if (row < 0) row += a.buckets;
+    }
+    pr = (const T*)a.table + (size_t)row * W;
+  }
+  float s = 0.f;
+  for (int c = tid; c < W; c += 256) {
+    float v = El<T>::ld(e + c) * a.scale;
+    if (pr) v += El<T>::ld(pr + c);
+    xs[c] = v;
+    s = fmaf(v, v, s);
+  }
+  float* x = a.x + (size_t)t * W;
+  if (!a.norm_w) {
+    for (int c = tid; c < W; c += 256) x[c] = xs[c];
+    return;
+  }
+  const float r = 1.f / sqrtf(block_sum_256(s, red) / (float)W + a.eps);
+  for (int c = tid; c < W; c += 256) x[c] = xs[c] * r * a.norm_w[c];
+}
+
+// ------------------------------------------------------------------------------------------------ seam of two sub-blocks (+ router)
+template <typename T>
+__global__ __launch_bounds__(256) void stk_sandwich_kernel(StkSandwichArgs a) {
+  extern __shared__ float lds[];
+  __shared__ float red[4];
+  float* xs = lds;             // [W]
+  float* zs = lds + a.W;       // [n_router]
+  const int t = blockIdx.x, W = a.W, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  float* x = a.x + (size_t)t * W;
+  if (a.post_w) {
+    float s = 0.f;
+    for (int c = tid; c < W; c += 256) {
+      float v = 0.f;
+      for (int j = 0; j < a.n1; j++) {
+        const size_t r = (size_t)t * a.n1 + j;
+        const float pv = a.p1[r * W + c];
+        v = a.pw ? fmaf(a.pw[r], pv, v) : v + pv;
+      }
+      v *= a.c1;
+      if (a.p2) v = fmaf(a.c2, a.p2[(size_t)t * W + c], v);
+      xs[c] = v;
+      s = fmaf(v, v, s);
+    }
+    const float r = 1.f / sqrtf(block_sum_256(s, red) / (float)W + a.eps);
+    for (int c = tid; c < W; c += 256) {
+      const float v = x[c] + xs[c] * r * a.post_w[c];
+      x[c] = v;
+      xs[c] = v;
+    }
+  } else {
+    for (int c = tid; c < W; c += 256) xs[c] = x[c];
+  }
+  if (!a.pre_w) return;
+  float s = 0.f;
+  for (int c = tid; c < W; c += 256) s = fmaf(xs[c], xs[c], s);
+  const float r = 1.f / sqrtf(block_sum_256(s, red) / (float)W + a.eps);
+  T* h = (T*)a.h + (size_t)t * W;
+  for (int c = tid; c < W; c += 256) {
+    const float v = xs[c] * r * a.pre_w[c];
+    xs[c] = v;
+    El<T>::st(h + c, v);
+  }
+  if (!a.router_w) return;
+  __syncthreads();
+  const T* rw = (const T*)a.router_w;
+  for (int e = wave; e < a.n_router; e += 4) {
+    float z = 0.f;
+    for (int c = lane; c < W; c += 64) z = fmaf(xs[c], El<T>::ld(rw + (size_t)e * W + c), z);
+    z = wave_sum(z);
+    if (lane == 0) zs[e] = z + (a.router_bias ? a.router_bias[e] : 0.f);
+  }
+  __syncthreads();
+  if (tid == 0) {
+    float zmax = -INFINITY, sum = 0.f;
+    for (int j = 0; j < a.top; j++) {
+      int best = -1;
+      float bz = -INFINITY;
+      for (int e = 0; e < a.n_router; e++) {
+        bool taken = false;
+        for (int q = 0; q < j; q++) taken = taken || a.pair_expert[(size_t)t * a.top + q] == e;
+        if (!taken && (best < 0 || zs[e] > bz)) best = e, bz = zs[e];
+      }
+      a.pair_expert[(size_t)t * a.top + j] = best;
+      if (j == 0) zmax = bz;  // (the first pick is the largest logit)
+      const float w = expf(bz - zmax);
+      a.pair_weight[(size_t)t * a.top + j] = w;
+      sum += w;
+    }
+    for (int j = 0; j < a.top; j++) a.pair_weight[(size_t)t * a.top + j] /= sum;
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ per-head norm, rotary, cache rows
+template <typename TO>
+__global__ __launch_bounds__(256) void stk_head_prep_kernel(StkHeadPrepArgs a) {
+  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, dim = a.dim;
+  const float* raw = a.raw + (size_t)t * a.ld;
+  const float p = (float)a.positions[t];
+  const int64_t slot = a.slots ? a.slots[t] : (int64_t)t;
+  const int rp = a.rot.pairs;
+  for (int hh = wave; hh < a.Hq + a.Hk; hh += 4) {
+    const bool is_q = hh < a.Hq;
+    const int h = is_q ? hh : hh - a.Hq;
+    if (!is_q && slot < 0) continue;
+    const float* src = raw + (is_q ? a.q_off : a.k_off) + h * dim;
+    const float* nw = is_q ? a.qn_w : a.kn_w;
+    float r = 1.f;
+    if (nw) {
+      float s = 0.f;
+      for (int c = lane; c < dim; c += 64) s = fmaf(src[c], src[c], s);
+      r = 1.f / sqrtf(wave_sum(s) / (float)dim + a.eps);
+    }
+    const float sc = is_q ? a.q_scale : a.k_scale;
+    TO* dst = is_q ? (TO*)a.q_out + (size_t)t * a.q_ld + h * dim : (TO*)a.k_out + (size_t)slot * a.k_ld + h * dim;
+    for (int c = lane; c < dim; c += 64) {
+      float v = nw ? src[c] * r * nw[c] : src[c];
+      if (c < 2 * rp) {
+        const int i = c < rp ? c : c - rp, oc = c < rp ? c + rp : c - rp;
+        const float o = nw ? src[oc] * r * nw[oc] : src[oc];
+        float cs, sn;
+        rot_cos_sin(a.rot, i, p, &cs, &sn);
+        v = c < rp ? v * cs - o * sn : v * cs + o * sn;
+      }
+      El<TO>::st(dst + c, v * sc);
+    }
+  }
+  if (a.v_out && slot >= 0) {
+    TO* dst = (TO*)a.v_out + (size_t)slot * a.v_ld;
+    for (int c = threadIdx.x; c < a.nv; c += 256) El<TO>::st(dst + c, raw[a.v_off + c]);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ inputs of the gated delta rule
+__global__ __launch_bounds__(256) void stk_delta_prep_kernel(StkDeltaPrepArgs a) {
+  extern __shared__ float lds[];
+  const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int H = a.H, G = a.G, dim = a.dim, vdim = a.vdim, nqk = G * dim, C = 2 * nqk + H * vdim, taps = a.taps;
+  float* ys = lds;  // [C] the convolved, activated row
+  const int b = seq_of_row(a.cu_q, a.B, t);
+  const int slot = a.state_slots[b];
+  if (slot < 0) return;
+  const int t0 = a.cu_q ? (int)a.cu_q[b] : t;
+  const int i = t - t0;                                   // place of the row in its sequence's part of the step
+  const bool fresh = a.positions[t0] == 0;                // the sequence starts in this step: nothing before its first row
+  const float* cs = a.conv_state + (size_t)slot * (taps - 1) * C;
+  for (int c = tid; c < C; c += 256) {
+    float y = 0.f;
+    for (int j = 0; j < taps; j++) {
+      const int e = i - (taps - 1) + j;
+      float in = 0.f;
+      if (e >= 0) in = a.raw[(size_t)(t0 + e) * a.ld + c];
+      else if (!fresh) in = cs[(size_t)(taps - 1 + e) * C + c];
+      y = fmaf(a.conv_w[(size_t)c * taps + j], in, y);
+    }
+    ys[c] = siluf_(y);
+  }
+  __syncthreads();
+  float* out = a.qkv_out + (size_t)t * C;
+  for (int hh = wave; hh < 2 * G; hh += 4) {  // q heads, then k heads: unit vectors
+    const float* src = ys + hh * dim;
+    float s = 0.f;
+    for (int c = lane; c < dim; c += 64) s = fmaf(src[c], src[c], s);
+    const float r = (hh < G ? a.q_scale : 1.f) / sqrtf(wave_sum(s) + 1e-6f);
+    for (int c = lane; c < dim; c += 64) out[hh * dim + c] = src[c] * r;
+  }
+  for (int c = tid; c < H * vdim; c += 256) out[2 * nqk + c] = ys[2 * nqk + c];
+  for (int h = tid; h < H; h += 256) a.beta_out[(size_t)t * H + h] = sigmoidf_(a.raw[(size_t)t * a.ld + C + h]);
+  for (int c = tid; c < H * dim; c += 256)
+    a.decay_out[(size_t)t * H * dim + c] = expf(-a.rate[c / dim] * softplusf_(a.raw2[(size_t)t * a.ld2 + c] + a.dt_bias[c]));
+}
+
+// the last taps - 1 inputs of every sequence of the step -> its slot (after the step's rows have read what the slot held)
+__global__ __launch_bounds__(256) void stk_conv_state_update_kernel(StkDeltaPrepArgs a) {
+  const int b = blockIdx.x;
+  const int slot = a.state_slots[b];
+  if (slot < 0) return;
+  const int C = 2 * a.G * a.dim + a.H * a.vdim, taps = a.taps;
+  const int t0 = a.cu_q ? (int)a.cu_q[b] : b, n = a.cu_q ? (int)a.cu_q[b + 1] - t0 : 1;
+  const bool fresh = a.positions[t0] == 0;
+  float* cs = a.conv_state + (size_t)slot * (taps - 1) * C;
+  for (int c = threadIdx.x; c < C; c += 256)
+    for (int r = 0; r < taps - 1; r++) {  // row r: the input taps - 1 - r places before the next token (rows are read above where they are written)
+      const int e = n - (taps - 1) + r;
+      float v = 0.f;
+      if (e >= 0) v = a.raw[(size_t)(t0 + e) * a.ld + c];
+      else if (!fresh) v = cs[(size_t)(taps - 1 + e) * C + c];
+      cs[(size_t)r * C + c] = v;
+    }
+}
+
+__global__ __launch_bounds__(256) void stk_sigmoid_pow_kernel(const float* z, int ldz, float* out, int ldo, int n, int64_t total, float inv_tau) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t t = i / n;
+    const int c = (int)(i % n);
+    out[t * ldo + c] = expf(-softplusf_(-z[t * ldz + c]) * inv_tau);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ the linear recurrence
+// A workgroup owns 256 / P columns of one head's state (a column = one value channel); a column's `dim` rows are spread over P
+// neighbouring lanes, R rows each, in registers for the whole step.  Sums over the rows (S^T k, S^T q) add a lane's R products in order,
+// then the P lanes by xor shuffles: an order fixed by `dim` alone.  q, k and the decays of TT tokens are staged in LDS once for all
+// columns.
+template <int R>
+__global__ __launch_bounds__(256) void stk_linear_scan_kernel(StkScanArgs a, int P) {
+  constexpr int TT = 16;
+  extern __shared__ float lds[];
+  const int dim = a.dim, vdim = a.vdim, dimP = P * R, CPB = 256 / P;
+  float* ks = lds;                   // [TT][dimP]
+  float* qs = ks + TT * dimP;        // [TT][dimP]
+  float* ds = qs + TT * dimP;        // [TT][dimP]
+  float* vs = ds + TT * dimP;        // [TT][CPB]
+  float* bs = vs + TT * CPB;         // [TT]
+  const int b = blockIdx.z, h = blockIdx.y, hq = h / a.qk_rep, tid = threadIdx.x;
+  const int slot = a.state_slots[b];
+  if (slot < 0) return;
+  const int r = tid % P, cl = tid / P, c = blockIdx.x * CPB + cl;
+  const bool col = c < vdim;
+  const int t0 = a.cu_q ? (int)a.cu_q[b] : b, n = a.cu_q ? (int)a.cu_q[b + 1] - t0 : 1;
+  const bool fresh = a.positions[t0] == 0;
+  float* sp = a.state + (((size_t)slot * a.H + h) * vdim + (col ? c : 0)) * dim + r * R;
+  float S[R];
+#pragma unroll
+  for (int j = 0; j < R; j++) S[j] = (!fresh && col && r * R + j < dim) ? sp[j] : 0.f;
+  const float hd = a.head_decay ? a.head_decay[h] : 1.f;
+  for (int i0 = 0; i0 < n; i0 += TT) {
+    const int nt = min(TT, n - i0);
+    __syncthreads();
+    for (int e = tid; e < nt * dimP; e += 256) {
+      const int i = e / dimP, d = e % dimP;
+      const size_t t = (size_t)(t0 + i0 + i);
+      const bool in = d < dim;
+      ks[e] = in ? a.k[t * a.ldk + hq * dim + d] : 0.f;
+      qs[e] = in ? a.q[t * a.ldq + hq * dim + d] * a.q_scale : 0.f;
+      if (a.decay) ds[e] = in ? a.decay[t * a.ldd + h * dim + d] : 1.f;
+    }
+    for (int e = tid; e < nt * CPB; e += 256) {
+      const int i = e / CPB, cc = blockIdx.x * CPB + e % CPB;
+      vs[e] = cc < vdim ? a.v[(size_t)(t0 + i0 + i) * a.ldv + h * vdim + cc] : 0.f;
+    }
+    if (a.beta)
+      for (int i = tid; i < nt; i += 256) bs[i] = a.beta[(size_t)(t0 + i0 + i) * a.ldb + h];
+    __syncthreads();
+    for (int i = 0; i < nt; i++) {
+      const float* kr = ks + i * dimP + r * R;
+      const float* qr = qs + i * dimP + r * R;
+      if (a.decay) {
+        const float* dr = ds + i * dimP + r * R;
+#pragma unroll
+        for (int j = 0; j < R; j++) S[j] *= dr[j];
+      } else {
+#pragma unroll
+        for (int j = 0; j < R; j++) S[j] *= hd;
+      }
+      float u = vs[i * CPB + cl];
+      if (a.beta) {
+        float dot = 0.f;
+#pragma unroll
+        for (int j = 0; j < R; j++) dot = fmaf(S[j], kr[j], dot);
+        for (int o = 1; o < P; o <<= 1) dot += __shfl_xor(dot, o, 64);
+        u = bs[i] * (u - dot);
+      }
+      float o_ = 0.f;
+#pragma unroll
+      for (int j = 0; j < R; j++) {
+        S[j] = fmaf(kr[j], u, S[j]);
+        o_ = fmaf(S[j], qr[j], o_);
+      }
+      for (int o = 1; o < P; o <<= 1) o_ += __shfl_xor(o_, o, 64);
+      if (r == 0 && col) a.out[(size_t)(t0 + i0 + i) * a.ldo + h * vdim + c] = o_;
+    }
+  }
+  if (col)
+#pragma unroll
+    for (int j = 0; j < R; j++)
+      if (r * R + j < dim) sp[j] = S[j];
+}
+
+// ------------------------------------------------------------------------------------------------ per-head output norm and gate
+template <typename T>
+__global__ __launch_bounds__(256) void stk_head_norm_gate_kernel(const float* o, const float* w, const float* gate, int gate_ld, int gate_act, float eps,
+                                                                 T* out, int H, int vdim) {
+  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int h = wave; h < H; h += 4) {
+    const float* src = o + ((size_t)t * H + h) * vdim;
+    float s = 0.f;
+    for (int c = lane; c < vdim; c += 64) s = fmaf(src[c], src[c], s);
+    const float r = 1.f / sqrtf(wave_sum(s) / (float)vdim + eps);
+    for (int c = lane; c < vdim; c += 64) {
+      float v = src[c] * r;
+      if (w) v *= w[c];
+      if (gate) {
+        const float g = gate[(size_t)t * gate_ld + h * vdim + c];
+        v *= gate_act == 1 ? siluf_(g) : sigmoidf_(g);
+      }
+      El<T>::st(out + ((size_t)t * H + h) * vdim + c, v);
+    }
+  }
+}
+
+}  // namespace
+
+// ================================================================================================ launchers
+void vra_stack_embed_pair(const StkEmbedPairArgs& a, int dtype, int64_t stream) {
+  VRA_CHECK_ARG(a.ids && a.positions && a.embed && a.x && a.T > 0 && a.W > 0 && a.V > 0, "stack embedding: null pointer or empty shape");
+  VRA_CHECK_ARG(!a.table || (a.buckets > 0 && a.prev_tokens && a.B > 0), "stack embedding: the pair table needs its bucket count and the previous tokens");
+  const size_t lds = (size_t)a.W * sizeof(float);
+  VRA_CHECK_ARG(lds <= 64 * 1024, "stack embedding: row does not fit LDS");
+  if (dtype == VRA_F32) launch_checked("stack embedding", [&] { stk_embed_pair_kernel<float><<<a.T, 256, lds, as_stream(stream)>>>(a); });
+  else launch_checked("stack embedding", [&] { stk_embed_pair_kernel<uint16_t><<<a.T, 256, lds, as_stream(stream)>>>(a); });
+}
+
+void vra_stack_sandwich_norm(const StkSandwichArgs& a, int dtype, int64_t stream) {
+  VRA_CHECK_ARG(a.x && a.T > 0 && a.W > 0 && (!a.post_w || (a.p1 && a.n1 >= 1)) && (!a.pre_w || a.h), "stack seam norm: null pointer or empty shape");
+  VRA_CHECK_ARG(!a.router_w || (a.pre_w && a.pair_expert && a.pair_weight && a.top >= 1 && a.top <= a.n_router), "stack seam norm: router outputs");
+  const size_t lds = ((size_t)a.W + a.n_router + 1) * sizeof(float);
+  VRA_CHECK_ARG(lds <= 64 * 1024, "stack seam norm: row does not fit LDS");
+  if (dtype == VRA_F32) launch_checked("stack seam norm", [&] { stk_sandwich_kernel<float><<<a.T, 256, lds, as_stream(stream)>>>(a); });
+  else launch_checked("stack seam norm", [&] { stk_sandwich_kernel<uint16_t><<<a.T, 256, lds, as_stream(stream)>>>(a); });
+}
+
+void vra_stack_head_prep(const StkHeadPrepArgs& a, int dtype, int64_t stream) {
+  VRA_CHECK_ARG(a.raw && a.positions && a.T > 0 && a.dim > 0 && a.Hq >= 0 && a.Hk >= 0 && (a.Hq == 0 || a.q_out) && (a.Hk == 0 || a.k_out),
+                "stack head prep: null pointer or empty shape");
+  VRA_CHECK_ARG(2 * a.rot.pairs <= a.dim && (a.rot.pairs == 0 || a.rot.freq_hi), "stack head prep: more rotated dimensions than the head has");
+  if (a.out_f32 || dtype == VRA_F32) launch_checked("stack head prep", [&] { stk_head_prep_kernel<float><<<a.T, 256, 0, as_stream(stream)>>>(a); });
+  else launch_checked("stack head prep", [&] { stk_head_prep_kernel<uint16_t><<<a.T, 256, 0, as_stream(stream)>>>(a); });
+}
+
+void vra_stack_delta_prep(const StkDeltaPrepArgs& a, int64_t stream) {
+  VRA_CHECK_ARG(a.raw && a.raw2 && a.conv_w && a.conv_state && a.rate && a.dt_bias && a.qkv_out && a.beta_out && a.decay_out && a.positions && a.state_slots,
+                "stack delta prep: null pointer");
+  VRA_CHECK_ARG(a.T > 0 && a.B > 0 && a.H > 0 && a.G > 0 && a.H % a.G == 0 && a.dim > 0 && a.vdim > 0 && a.taps >= 1, "stack delta prep: shapes");
+  const size_t lds = ((size_t)2 * a.G * a.dim + (size_t)a.H * a.vdim) * sizeof(float);
+  VRA_CHECK_ARG(lds <= 64 * 1024, "stack delta prep: row does not fit LDS");
+  launch_checked("stack delta prep", [&] { stk_delta_prep_kernel<<<a.T, 256, lds, as_stream(stream)>>>(a); });
+}
+
+void vra_stack_conv_state_update(const StkDeltaPrepArgs& a, int64_t stream) {
+  VRA_CHECK_ARG(a.raw && a.conv_state && a.positions && a.state_slots && a.B > 0 && a.taps >= 1, "stack conv state: null pointer or empty shape");
+  if (a.taps < 2) return;
+  launch_checked("stack conv state", [&] { stk_conv_state_update_kernel<<<a.B, 256, 0, as_stream(stream)>>>(a); });
+}
+
+void vra_stack_sigmoid_pow(const float* z, int ldz, float* out, int ldo, int T, int n, float inv_tau, int64_t stream) {
+  VRA_CHECK_ARG(z && out && T > 0 && n > 0, "stack decay: null pointer or empty shape");
+  const int64_t total = (int64_t)T * n;
+  const int grid = (int)std::min<int64_t>((total + 255) / 256, 4096);
+  launch_checked("stack decay", [&] { stk_sigmoid_pow_kernel<<<grid, 256, 0, as_stream(stream)>>>(z, ldz, out, ldo, n, total, inv_tau); });
+}
+
+void vra_stack_linear_scan(const StkScanArgs& a, int64_t stream) {
+  VRA_CHECK_ARG(a.q && a.k && a.v && a.state && a.state_slots && a.positions && a.out && (a.decay || a.head_decay), "stack linear scan: null pointer");
+  VRA_CHECK_ARG(a.B > 0 && a.H > 0 && a.qk_rep >= 1 && a.H % a.qk_rep == 0 && a.dim > 0 && a.dim <= 256 && a.vdim > 0, "stack linear scan: key size at most 256");
+  constexpr int R = 8;
+  int P = 1;
+  while (P * R < a.dim) P <<= 1;
+  const int CPB = 256 / P, dimP = P * R;
+  const size_t lds = ((size_t)16 * dimP * 3 + (size_t)16 * CPB + 16) * sizeof(float);
+  dim3 grid((a.vdim + CPB - 1) / CPB, a.H, a.B);
+  launch_checked("stack linear scan", [&] { stk_linear_scan_kernel<R><<<grid, 256, lds, as_stream(stream)>>>(a, P); });
+}
+
+void vra_stack_head_norm_gate(const float* o, const float* w, const float* gate, int gate_ld, int gate_act, float eps, void* out, int T, int H, int vdim,
+                              int dtype, int64_t stream) {
+  VRA_CHECK_ARG(o && out && T > 0 && H > 0 && vdim > 0, "stack head norm: null pointer or empty shape");
+  if (dtype == VRA_F32)
+    launch_checked("stack head norm", [&] { stk_head_norm_gate_kernel<float><<<T, 256, 0, as_stream(stream)>>>(o, w, gate, gate_ld, gate_act, eps, (float*)out, H, vdim); });
+  else
+    launch_checked("stack head norm", [&] {
+      stk_head_norm_gate_kernel<uint16_t><<<T, 256, 0, as_stream(stream)>>>(o, w, gate, gate_ld, gate_act, eps, (uint16_t*)out, H, vdim);
+    });
+}

@@ -73,7 +73,8 @@ TINYLLAMA = dict(arch="llama", hidden_size=2048, intermediate_size=5632, num_lay
 class Engine:
     def __init__(self, cfg, *, block_size=64, max_num_seqs=32, max_model_len=0, num_gpu_blocks=0, kv_fraction=0.0,
                  prefill_chunk=8192, enable_prefix_cache=False, use_graph=True, tp_rank=0, tp_world_size=1, device=0,
-                 seed=1234, comm=None, fp8_kvcache=False, cpu_mem_fold=0.0, swap_cooling_ms=0, min_tokens_left_for_swap=0):
+                 seed=1234, comm=None, fp8_kvcache=False, cpu_mem_fold=0.0, swap_cooling_ms=0, min_tokens_left_for_swap=0,
+                 num_state_slots=0):
         # cpu_mem_fold: CPU swap space as a fraction of the KV blocks, PINNED per layer at finalize.  0 (no swap space: preempted
         # sequences are recomputed) unless the caller asks — the reference's default 0.2 (kvcache_allocator.rs:317) is applied where
         # the reference's ENGINE plans CPU block ids, i.e. on the runner-IPC path (runner_ipc.py, host/runner_main.cpp); as the
@@ -88,7 +89,8 @@ class Engine:
                                enable_prefix_cache=int(enable_prefix_cache), prefix_cache_fraction=0.65,
                                use_graph=int(use_graph), tp_rank=tp_rank, tp_world_size=tp_world_size, device=device,
                                seed=seed, fp8_kvcache=int(fp8_kvcache), cpu_mem_fold=cpu_mem_fold,
-                               swap_cooling_ms=swap_cooling_ms, min_tokens_left_for_swap=min_tokens_left_for_swap)
+                               swap_cooling_ms=swap_cooling_ms, min_tokens_left_for_swap=min_tokens_left_for_swap,
+                               num_state_slots=num_state_slots)
         if self.mc.arch == 3:
             if max_model_len > 0:  # a layer stack has no position table: the longest sequence is what the engine is asked to hold
                 self.mc.max_position_embeddings = max_model_len

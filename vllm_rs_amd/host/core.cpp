@@ -217,7 +217,15 @@ int BlockManager::required_blocks(const Sequence& s) {
   }
   return s.num_blocks();
 }
-bool BlockManager::can_allocate(const Sequence& s) { return free_count_ >= required_blocks(s); }
+bool BlockManager::can_allocate(const Sequence& s) {
+  if (slots_.enabled() && slots_.slot_of(s.id) < 0 && slots_.num_free() == 0) return false;
+  return free_count_ >= required_blocks(s);
+}
+bool BlockManager::take_slot(Sequence& s) {
+  if (!slots_.enabled()) return true;
+  s.state_slot = slots_.acquire(s.id);
+  return s.state_slot >= 0;
+}
 bool BlockManager::allocate_fresh(Sequence& s) {
   s.num_cached_tokens = 0;
   const int need = s.num_blocks();
@@ -256,11 +264,13 @@ bool BlockManager::allocate_with_prefix(Sequence& s) {  // :346-442
   return true;
 }
 bool BlockManager::allocate(Sequence& s) {
-  if (cache_.enabled()) return allocate_with_prefix(s);
-  return allocate_fresh(s);
+  if (slots_.enabled() && slots_.slot_of(s.id) < 0 && slots_.num_free() == 0) return false;
+  if (!(cache_.enabled() ? allocate_with_prefix(s) : allocate_fresh(s))) return false;
+  return take_slot(s);
 }
 void BlockManager::deallocate(const Sequence& s) {
   for (auto it = s.block_table.rbegin(); it != s.block_table.rend(); ++it) decrement_ref((int)*it);
+  slots_.release(s.id);
 }
 bool BlockManager::can_append(const Sequence& s) const {
   int need = 1;
@@ -304,6 +314,7 @@ bool BlockManager::can_swap_out(const Sequence& s) const {
 }
 bool BlockManager::can_swap_in(const Sequence& s) const { return free_count_ > s.num_blocks(); }
 bool BlockManager::ensure_allocate(Sequence& s) {
+  if (!take_slot(s)) return false;
   while ((int)s.block_table.size() < s.num_blocks()) {
     const int id = pop_front();
     if (id < 0) return false;

@@ -37,6 +37,8 @@ struct Sequence {
   std::vector<uint32_t> block_table;
   int num_cached_tokens = 0;
   int block_size = 64;
+  // slot of this sequence's recurrent state (models whose layers carry a state from token to token: StateSlots below); -1 = none
+  int state_slot = -1;
   uint32_t last_token = 0;
   int prompt_len = 0;
   // SamplingParams (config.rs:476-520) as ModelRunner::sample reads them (runner.rs:1405-1497); "None" = unset:
@@ -106,6 +108,47 @@ class PrefixCache {
   uint64_t access_counter_ = 0;
 };
 
+// Slots for what a model carries from token to token beside the paged cache (matrix states of linear-attention layers, the last inputs
+// of short convolutions, the previous token): one slot per live sequence, taken when the sequence gets its blocks, given back with
+// them.  A freed slot is the next one handed out (LIFO); nothing is cleared on the host or the device: a sequence that starts at
+// position 0 starts from a zero state inside the kernels.
+class StateSlots {
+ public:
+  void reset(int n) {
+    free_.clear();
+    owner_.clear();
+    total_ = n > 0 ? n : 0;
+    for (int i = total_ - 1; i >= 0; i--) free_.push_back(i);
+  }
+  bool enabled() const { return total_ > 0; }
+  int total() const { return total_; }
+  int num_free() const { return (int)free_.size(); }
+  int slot_of(int64_t seq) const {
+    auto it = owner_.find(seq);
+    return it == owner_.end() ? -1 : it->second;
+  }
+  int acquire(int64_t seq) {  // the sequence's slot, a new one if it holds none; -1: none left
+    auto it = owner_.find(seq);
+    if (it != owner_.end()) return it->second;
+    if (free_.empty()) return -1;
+    const int s = free_.back();
+    free_.pop_back();
+    owner_[seq] = s;
+    return s;
+  }
+  void release(int64_t seq) {
+    auto it = owner_.find(seq);
+    if (it == owner_.end()) return;
+    free_.push_back(it->second);
+    owner_.erase(it);
+  }
+
+ private:
+  int total_ = 0;
+  std::vector<int> free_;
+  std::unordered_map<int64_t, int> owner_;
+};
+
 // src/core/block_manager.rs (GPU blocks only)
 class BlockManager {
  public:
@@ -134,8 +177,13 @@ class BlockManager {
   bool swap_in(const Sequence& s, std::vector<std::pair<int, int>>* cpu_to_gpu);   // :957-995 (blocks pre-allocated)
   void free_cpu_swap_for_seq(int64_t seq_id);   // :997-1007
   int evict_prefix_cache_until_free(int required_free);
+  // state slots ride with the blocks: allocate / ensure_allocate take one for the sequence (and fail without one), deallocate frees it
+  void set_state_slots(int n) { slots_.reset(n); }
+  const StateSlots& state_slots() const { return slots_; }
 
  private:
+  bool take_slot(Sequence& s);
+  StateSlots slots_;
   int pop_front();
   void push_back(int id);
   void unlink(int id);

@@ -124,7 +124,7 @@ class Engine {
   uint8_t* h_meta_ = nullptr;
   uint8_t* d_meta_ = nullptr;
   size_t meta_bytes_ = 0;
-  size_t off_ids_, off_pos_, off_slots_, off_bt_, off_ctx_, off_cuq_, off_last_, off_dids_, off_dpos_, off_dslots_, off_rows_;
+  size_t off_ids_, off_pos_, off_slots_, off_bt_, off_ctx_, off_cuq_, off_last_, off_dids_, off_dpos_, off_dslots_, off_rows_, off_state_, off_prev_;
   uint32_t* d_tokens_ = nullptr;
   uint32_t* h_tokens_ = nullptr;
   uint32_t* h_err_ = nullptr;  // pinned copy of the device error words (split-K exchange, one-shot all-reduce), read every step
@@ -211,6 +211,7 @@ class Engine {
     // CPU swap space (kvcache_allocator.rs:673): num_cpu_blocks = gpu blocks x cpu_mem_fold
     num_cpu_blocks_ = ec_.cpu_mem_fold > 0.f ? (int)((double)nb * ec_.cpu_mem_fold) : 0;
     bm_.reset(new BlockManager((int)nb, ec_.block_size, ec_.enable_prefix_cache != 0, ec_.prefix_cache_fraction, num_cpu_blocks_));
+    if (model_ && model_->state_bytes_per_slot() > 0) bm_->set_state_slots(num_state_slots());
     SchedulerConfig sc;
     if (ec_.swap_cooling_ms) sc.swap_cooling_ms = std::max(0, ec_.swap_cooling_ms);
     if (ec_.min_tokens_left_for_swap) sc.min_tokens_left_for_swap = std::max(0, ec_.min_tokens_left_for_swap);
@@ -232,6 +233,8 @@ class Engine {
     off_dids_ = o, o += al(B * 4);
     off_dpos_ = o, o += al(B * 8);
     off_dslots_ = o, o += al(B * 8);
+    off_state_ = o, o += al(B * 4);
+    off_prev_ = o, o += al(B * 4);
     off_bt_ = o, o += al(B * (size_t)max_blocks_per_seq_ * 4);
     off_ids_ = o, o += al(T * 4);
     off_pos_ = o, o += al(T * 8);
@@ -266,6 +269,8 @@ class Engine {
     prepared_ = true;
     return true;
   }
+  // state slots of a model that carries a state per sequence: as many as the scheduler may batch unless the caller asks for fewer
+  int num_state_slots() const { return ec_.num_state_slots > 0 ? ec_.num_state_slots : max_seqs_; }
   bool finalize() {
     if (dry()) return finalize_dry();
     if (model_->world() > 1 && !model_->has_comm()) return fail("tensor parallel world_size > 1 without a communicator (vra_engine_set_comm before finalize)");
@@ -276,6 +281,11 @@ class Engine {
     if (nb < 2) return fail("not enough memory for the KV cache");
     if (nb > (1 << 24)) nb = 1 << 24;
     if (!model_->init_kv_cache((int)nb)) return fail("kv cache: " + model_->error);
+    if (model_->state_bytes_per_slot() > 0) {
+      // a cached prefix or a swapped-out block holds keys and values only: the state a sequence had after those tokens is not kept
+      if (ec_.enable_prefix_cache || ec_.cpu_mem_fold > 0.f) return fail("a model with a per-sequence state runs without prefix cache and CPU swap space");
+      if (!model_->init_state(num_state_slots())) return fail("state slots: " + model_->error);
+    }
     setup_host(nb);
     if (num_cpu_blocks_ > 0) {  // pinned host copies of whole blocks, per layer: K then V (kvcache_allocator.rs:905-930)
       h_swap_k_.assign(model_->kv_layers(), nullptr);
@@ -317,6 +327,7 @@ class Engine {
     uint32_t* h_ctx = (uint32_t*)(h_meta_ + off_ctx_);
     uint32_t* h_cuq = (uint32_t*)(h_meta_ + off_cuq_);
     uint32_t* h_last = (uint32_t*)(h_meta_ + off_last_);
+    int32_t* h_state = (int32_t*)(h_meta_ + off_state_);
     const int BS = ec_.block_size, CHUNK = ec_.prefill_chunk;
     int T = 0, max_q = 0, max_ctx = 0, max_bt = 0;
     InputMetadata md;
@@ -352,6 +363,8 @@ class Engine {
         done += take;
       }
       h_ctx[b] = (uint32_t)(s.num_cached_tokens + n);
+      h_state[b] = s.state_slot;
+      ((uint32_t*)(h_meta_ + off_prev_))[b] = s.num_cached_tokens > 0 ? s.token_ids[s.num_cached_tokens - 1] : 0u;
       for (int j = 0; j < max_bt; j++) h_bt[b * (size_t)max_bt + j] = j < (int)s.block_table.size() ? s.block_table[j] : 0;
       T += n;
       h_cuq[b + 1] = (uint32_t)T;
@@ -377,9 +390,12 @@ class Engine {
     int64_t* h_slots = (int64_t*)(h_meta_ + off_dslots_);
     uint32_t* h_bt = (uint32_t*)(h_meta_ + off_bt_);
     uint32_t* h_ctx = (uint32_t*)(h_meta_ + off_ctx_);
+    int32_t* h_state = (int32_t*)(h_meta_ + off_state_);
     const int BS = ec_.block_size, stride = max_blocks_per_seq_;
     int max_ctx = 0;
     for (int b = 0; b < bucket; b++) {
+      h_state[b] = b < (int)ids.size() ? run[ids[b]].state_slot : -1;
+      ((uint32_t*)(h_meta_ + off_prev_))[b] = b < (int)ids.size() && run[ids[b]].len() >= 2 ? run[ids[b]].token_ids[run[ids[b]].len() - 2] : 0u;
       if (b < (int)ids.size()) {
         const Sequence& s = run[ids[b]];
         h_ids[b] = s.last_token;
@@ -414,6 +430,8 @@ class Engine {
     md.context_lens = (const uint32_t*)(d_meta_ + off_ctx_);
     md.cu_seqlens_q = (const uint32_t*)(d_meta_ + off_cuq_);
     md.last_token_rows = (const uint32_t*)(d_meta_ + off_last_);
+    md.state_slots = (const int32_t*)(d_meta_ + off_state_);
+    md.prev_tokens = (const uint32_t*)(d_meta_ + off_prev_);
   }
   // one H2D copy per step (the reference does five, runner.rs:1222-1238): a decode step only needs the head of the staging
   // buffer (per-sequence arrays + the block-table rows in use), a prefill step everything up to its last token
@@ -1074,10 +1092,16 @@ struct RawSampling {
 static int32_t forward_raw_impl(Engine* en, const uint32_t* h_ids, const int64_t* h_positions, const int64_t* h_slot_mapping,
                                 int32_t n_tokens, int32_t is_prefill, const uint32_t* h_block_tables, int32_t max_blocks,
                                 const uint32_t* h_context_lens, const uint32_t* h_cu_seqlens_q, int32_t n_seqs,
-                                float* h_logits_out, uint32_t* h_tokens_out, const RawSampling* smp, const uint32_t* h_rows = nullptr, int32_t n_rows = 0) {
+                                float* h_logits_out, uint32_t* h_tokens_out, const RawSampling* smp, const uint32_t* h_rows = nullptr, int32_t n_rows = 0,
+                                const int32_t* h_state = nullptr, const uint32_t* h_prev = nullptr) {
   if (!en->sched_) {
     en->error = "engine not finalised";
     return -1;
+  }
+  if (en->model_->state_bytes_per_slot() > 0) {
+    if (!h_state) return en->error = "forward_raw: this model keeps a state per sequence; its steps go through the scheduler or replay_step", -1;
+    for (int b = 0; b < n_seqs; b++)
+      if (h_state[b] < 0 || h_state[b] >= en->num_state_slots()) return en->error = "forward_raw: state slot outside the pool", -1;
   }
   if (n_tokens > std::max(en->max_step_tokens_, en->max_seqs_) || n_seqs > en->max_seqs_ || max_blocks > en->max_blocks_per_seq_) {
     en->error = "forward_raw: batch exceeds engine limits";
@@ -1134,6 +1158,10 @@ static int32_t forward_raw_impl(Engine* en, const uint32_t* h_ids, const int64_t
     for (int b = 0; b < n_seqs; b++) memcpy(en->h_meta_ + en->off_bt_ + (size_t)b * bt_stride * 4, h_block_tables + (size_t)b * max_blocks, (size_t)max_blocks * 4);
   }
   memcpy(en->h_meta_ + en->off_ctx_, h_context_lens, (size_t)n_seqs * 4);
+  for (int b = 0; b < std::max(bucket, (int)n_seqs) && b < en->max_seqs_; b++) {
+    ((int32_t*)(en->h_meta_ + en->off_state_))[b] = h_state && b < n_seqs ? h_state[b] : -1;
+    ((uint32_t*)(en->h_meta_ + en->off_prev_))[b] = h_prev && b < n_seqs ? h_prev[b] : 0u;
+  }
   for (int b = n_seqs; b < bucket && graph_decode; b++) {
     ((uint32_t*)(en->h_meta_ + en->off_dids_))[b] = 0;
     ((int64_t*)(en->h_meta_ + en->off_dpos_))[b] = 0;
@@ -1260,7 +1288,7 @@ extern "C" int32_t vra_engine_replay_step(void* e, int32_t n_entries, const int6
     if (s.len() + h_counts[i] > en->max_model_len_) return en->error = "replay_step: request longer than max_model_len", -1;
     decode = decode && h_counts[i] == 1 && s.num_cached_tokens > 0;
     s.token_ids.insert(s.token_ids.end(), h_tokens + T, h_tokens + T + h_counts[i]);
-    if (!en->bm_->ensure_allocate(s)) return en->error = "replay_step: no free KV block (the pool is smaller than the live requests need)", -1;
+    if (!en->bm_->ensure_allocate(s)) return en->error = "replay_step: no free KV block or state slot (the pool is smaller than the live requests need)", -1;
     seqs.push_back(&s);
     T += h_counts[i];
     for (int j = 0; j < h_n_want[i]; j++)
@@ -1272,9 +1300,13 @@ extern "C" int32_t vra_engine_replay_step(void* e, int32_t n_entries, const int6
     for (auto* s : seqs) max_bt = std::max(max_bt, (int)s->block_table.size());
     std::vector<uint32_t> ids(T), bt((size_t)n_entries * max_bt, 0), ctx(n_entries), cu(n_entries + 1, 0), rows;
     std::vector<int64_t> pos(T), slots(T);
+    std::vector<int32_t> state(n_entries, -1);
+    std::vector<uint32_t> prev(n_entries, 0);
     int t = 0, w = 0;
     for (int i = 0; i < n_entries; i++) {
       const vra::Sequence& s = *seqs[i];
+      state[i] = s.state_slot;
+      if (s.num_cached_tokens > 0) prev[i] = s.token_ids[s.num_cached_tokens - 1];
       for (int p = s.num_cached_tokens; p < s.len(); p++, t++) {
         ids[t] = s.token_ids[p], pos[t] = p;
         slots[t] = (int64_t)s.block_table[p / BS] * BS + p % BS;
@@ -1294,7 +1326,7 @@ extern "C" int32_t vra_engine_replay_step(void* e, int32_t n_entries, const int6
       rows.assign(1, 0);
     }
     if (forward_raw_impl(en, ids.data(), pos.data(), slots.data(), T, decode ? 0 : 1, bt.data(), max_bt, ctx.data(), decode ? nullptr : cu.data(), n_entries, out,
-                         nullptr, nullptr, rows.data(), (int32_t)rows.size()) != 0)
+                         nullptr, nullptr, rows.data(), (int32_t)rows.size(), en->model_->state_bytes_per_slot() > 0 ? state.data() : nullptr, prev.data()) != 0)
       return -1;
     for (auto* s : seqs) s->num_cached_tokens = s->len();
   }

@@ -30,6 +30,11 @@ struct InputMetadata {
   // sequence of a prefill step, every row of a decode step
   const uint32_t* logit_rows = nullptr;  // [n_logit_rows]
   int n_logit_rows = 0;
+  // slot of every sequence's recurrent state (models with state_bytes_per_slot() > 0); -1: a padded lane, nothing read or written.
+  // A sequence whose first token of the step stands at position 0 starts from a zero state whatever its slot holds.
+  const int32_t* state_slots = nullptr;  // [B]
+  // the token before each sequence's first row of the step (models that embed token pairs); unused at position 0
+  const uint32_t* prev_tokens = nullptr;  // [B]
 };
 
 class ModelBase {
@@ -50,6 +55,10 @@ class ModelBase {
   virtual void* v_cache(int l) const = 0;
   // bytes of ONE block over all layers, K and V (the engine plans the block count from free memory with it)
   virtual int64_t kv_bytes_per_block() const = 0;
+  // what the model carries from token to token for ONE sequence beside the paged cache, in bytes (0: nothing); the engine hands out
+  // `slots` slots through its block manager (core.h StateSlots) and names each sequence's slot in InputMetadata::state_slots
+  virtual int64_t state_bytes_per_slot() const { return 0; }
+  virtual bool init_state(int /*slots*/) { return true; }
   virtual bool init_buffers(int max_tokens, int max_seqs) = 0;
   // rows of logits one forward can leave (>= max_seqs)
   virtual int max_logit_rows() const = 0;

@@ -60,21 +60,39 @@ bool StackModel::parse_spec(const char* spec) {
       width_ = (int)num("width", 0), vocab_ = (int)num("vocab", 0), groups_ = (int)num("groups", 1);
       eps_ = (float)num("eps", 1e-6), residual_mult_ = (float)num("residual_mult", 1.0), logit_scale_ = (float)num("logit_scale", 1.0);
       pos_base_ = num("pos_base", 10000.0);
-      auto pick = [&](const char* k, const char* a, const char* b, int* out) {
+      auto pick = [&](const char* k, const char* a, const char* b, int* out, const char* c = nullptr) {
         const std::string v = f.count(k) ? f[k] : a;
-        if (v != a && v != b) return spec_error_ = std::string("layer stack spec: ") + k + " must be " + a + " or " + b, false;
-        *out = v == b;
+        if (v != a && v != b && !(c && v == c)) return spec_error_ = std::string("layer stack spec: ") + k + " must be " + a + " or " + b + (c ? std::string(" or ") + c : ""), false;
+        *out = v == b ? 1 : (c && v == c ? 2 : 0);
         return true;
       };
-      if (!pick("block", "parallel", "sequential", &block_) || !pick("norm", "rms", "dyt", &norm_kind_) || !pick("pos", "sinusoid", "none", &pos_kind_)) return false;
+      if (!pick("block", "parallel", "sequential", &block_, "sandwich") || !pick("norm", "rms", "dyt", &norm_kind_) || !pick("pos", "sinusoid", "none", &pos_kind_))
+        return false;
+      norm_offset_ = (float)num("norm_offset", 0.0), embed_scale_ = (float)num("embed_scale", 1.0), embed_norm_ = (int)num("embed_norm", 0);
+      pair_buckets_ = (int)num("pair_buckets", 0), pair_mul_prev_ = (int64_t)num("pair_mul_prev", 0), pair_mul_cur_ = (int64_t)num("pair_mul_cur", 0);
     } else if (kind == "layer") {
       StackLayer L;
       L.heads = (int)num("heads", 0), L.kv_heads = (int)num("kv_heads", L.heads), L.dim = (int)num("dim", 0), L.vdim = (int)num("vdim", L.dim);
       L.scale = (float)num("scale", L.dim > 0 ? 1.0 / sqrt((double)L.dim) : 1.0), L.softcap = (float)num("softcap", 0.0);
       L.temp_coef = (float)num("temp_coef", 0.0), L.temp_every = (int)num("temp_every", 0), L.kv_from = (int)num("kv_from", -1);
       const std::string mix = f.count("mixer") ? f["mixer"] : "attention";
-      L.mixer = mix == "latent" ? 1 : (mix == "sigmoid" ? 2 : 0);
-      if (mix != "attention" && mix != "latent" && mix != "sigmoid") return spec_error_ = "layer stack spec: unknown mixer " + mix, false;
+      L.mixer = mix == "latent" ? 1 : (mix == "sigmoid" ? 2 : (mix == "delta" ? 3 : (mix == "retention" ? 4 : (mix == "parallel" ? 5 : 0))));
+      if (mix != "attention" && L.mixer == 0) return spec_error_ = "layer stack spec: unknown mixer " + mix, false;
+      L.conv = (int)num("conv", 0), L.rank_a = (int)num("rank_a", 0), L.rank_g = (int)num("rank_g", 0), L.chunk = (int)num("chunk", 0);
+      L.qk_norm = (int)num("qk_norm", 0), L.has_bias = (int)num("bias", 0);
+      L.rs_factor = num("rs_factor", 0.0), L.rs_low = num("rs_low", 1.0), L.rs_high = num("rs_high", 4.0), L.rs_original = num("rs_original", 0.0);
+      L.r_heads = (int)num("r_heads", 0), L.r_dim = (int)num("r_dim", 0), L.r_vdim = (int)num("r_vdim", L.r_dim), L.tau = (float)num("tau", 1.0);
+      L.left_scale = (float)num("left_scale", 1.0), L.right_scale = (float)num("right_scale", 1.0);
+      if (f.count("decay")) {
+        std::istringstream ds(f["decay"]);
+        std::string item;
+        while (std::getline(ds, item, ',')) L.decay.push_back((float)strtod(item.c_str(), nullptr));
+      }
+      {
+        const std::string rk = f.count("router") ? f["router"] : "sigmoid", ak = f.count("act") ? f["act"] : "clamped";
+        if ((rk != "sigmoid" && rk != "softmax") || (ak != "clamped" && ak != "silu")) return spec_error_ = "layer stack spec: router is sigmoid or softmax, act clamped or silu", false;
+        L.router_kind = rk == "softmax", L.act_kind = ak == "silu" ? 2 : 0;
+      }
       L.weights_of = (int)num("weights_of", -1);
       L.rot_dim = (int)num("rot_dim", 0), L.kv_rank = (int)num("kv_rank", 0), L.q_rank = (int)num("q_rank", 0), L.rot_dims = (int)num("rot_dims", L.rot_dim);
       L.sink = (int)num("sink", 0), L.rot_base = num("rot_base", 10000.0), L.yarn_factor = num("yarn_factor", 0.0);
@@ -99,8 +117,18 @@ bool StackModel::parse_spec(const char* spec) {
     const std::string at = " (layer " + std::to_string(i) + ")";
     if (L.heads <= 0 || L.kv_heads <= 0 || L.heads % L.kv_heads || L.dim <= 0 || L.vdim <= 0 || (L.mixer == 0 && L.vdim > 256))
       return spec_error_ = "layer stack spec: heads must be a multiple of kv_heads, sizes positive, value size at most 256" + at, false;
-    if (L.mixer != 0 && block_ != 1) return spec_error_ = "layer stack spec: latent and sigmoid mixers run in sequential blocks" + at, false;
+    if ((L.mixer == 1 || L.mixer == 2) && block_ != 1) return spec_error_ = "layer stack spec: latent and sigmoid mixers run in sequential blocks" + at, false;
     if (L.mixer == 0 && block_ != 0) return spec_error_ = "layer stack spec: the softmax mixer with temperature and cap runs in parallel blocks" + at, false;
+    if (L.mixer >= 3 && block_ != 2) return spec_error_ = "layer stack spec: delta, retention and parallel mixers run in sandwich blocks" + at, false;
+    if (block_ == 2 && (L.mixer < 3 || (L.mlp != 0 && L.mlp != 2) || L.weights_of >= 0))
+      return spec_error_ = "layer stack spec: sandwich blocks hold delta, retention or parallel mixers and a mixture of experts or no feed-forward" + at, false;
+    if (L.mixer == 3 && (L.conv < 1 || L.rank_a < 1 || L.rank_g < 1 || L.dim > 256)) return spec_error_ = "layer stack spec: the delta mixer needs conv >= 1, rank_a, rank_g, dim <= 256" + at, false;
+    if (L.mixer == 4 && ((int)L.decay.size() != L.heads || L.kv_heads != L.heads || L.rot_dims < 0 || L.rot_dims > L.dim || L.rot_dims % 2 || L.dim > 256))
+      return spec_error_ = "layer stack spec: retention needs one decay per head, kv_heads = heads, an even rot_dims <= dim <= 256" + at, false;
+    if (L.mixer == 5 && (L.r_heads <= 0 || L.r_dim <= 0 || L.r_dim > 256 || L.r_vdim <= 0 || L.rank_a < 1 || !(L.tau > 0.f) || L.rot_dims < 0 || L.rot_dims > L.dim || L.rot_dims % 2 ||
+                         L.chunk < 0 || L.vdim > 256 || (L.rs_factor > 0.0 && (L.rs_original <= 0.0 || L.rs_high <= L.rs_low))))
+      return spec_error_ = "layer stack spec: the parallel mixer needs r_heads, r_dim <= 256, r_vdim, rank_a, tau > 0, an even rot_dims <= dim, vdim <= 256" + at, false;
+    if (L.router_kind == 1 && (block_ != 2 || L.shared_ff > 0)) return spec_error_ = "layer stack spec: the softmax router belongs to sandwich blocks and has no shared expert" + at, false;
     if (L.mixer != 0 && L.kv_from >= 0) return spec_error_ = "layer stack spec: kv_from belongs to the softmax mixer" + at, false;
     if (L.mixer == 1 && (L.kv_rank <= 0 || L.q_rank <= 0 || L.rot_dim < 0 || L.kv_rank > 256 || L.rot_dims < 0 || L.rot_dims > L.rot_dim || L.rot_dims % 2 ||
                          (L.yarn_factor > 0.0 && (L.yarn_original <= 0.0 || L.yarn_fast <= 0.0 || L.yarn_slow <= 0.0))))
@@ -117,7 +145,9 @@ bool StackModel::parse_spec(const char* spec) {
           S.kv_rank != L.kv_rank || S.q_rank != L.q_rank || S.mlp != L.mlp || S.ff != L.ff || S.kv_from >= 0 || L.kv_from >= 0)
         return spec_error_ = "layer stack spec: a layer that shares weights has the shapes of the layer it names" + at, false;
     }
-    if (L.kv_from >= 0) {
+    if (!L.has_cache()) {
+      if (L.kv_from >= 0) return spec_error_ = "layer stack spec: kv_from belongs to the softmax mixer" + at, false;
+    } else if (L.kv_from >= 0) {
       if (L.kv_from >= (int)i) return spec_error_ = "layer stack spec: kv_from must name an earlier layer" + at, false;
       const StackLayer& S = layers_[L.kv_from];
       if (!S.owns_cache || S.kv_heads != L.kv_heads || S.dim != L.dim || S.vdim != L.vdim)
@@ -128,6 +158,7 @@ bool StackModel::parse_spec(const char* spec) {
       L.cache = (int)cache_layer_.size();
       cache_layer_.push_back((int)i);
     }
+    if (!L.has_cache()) L.owns_cache = false;  // (their past lives in the state slot; the cache entry keeps the tables uniform and holds no bytes)
     if (L.mlp == 1 && L.ff <= 0) return spec_error_ = "layer stack spec: dense feed-forward without ff" + at, false;
     if (L.mlp == 2 && (L.ff <= 0 || L.experts <= 0 || L.top < 1 || L.top > L.experts))
       return spec_error_ = "layer stack spec: mixture of experts needs ff, experts and 1 <= top <= experts" + at, false;
@@ -274,14 +305,108 @@ bool StackModel::finalize_weights() {
       out->push_back(v);
     }
   };
-  if (!up_mat("embed", vocab_, W, &embed_) || !up_mat("head", vocab_, W, &head_) || !up_norm("final.norm", &final_norm_, &final_b_, &final_alpha_)) return false;
+  // a norm weight stored around zero: the offset is added once, here
+  auto up_norm_off = [&](const std::string& name, int64_t n, float** w) {
+    const HostTensor* t;
+    if (!need(name, n, -1, &t)) return false;
+    std::vector<float> v;
+    f32_of(*t, &v);
+    for (float& e : v) e += norm_offset_;
+    return (*w = upload_floats(v)) != nullptr;
+  };
+  // the shape a staged tensor came with (sizes the config does not carry: the ranks of low-rank projections)
+  auto rows_of = [&](const std::string& name, int64_t cols) -> int64_t {
+    auto it = staged_.find(name);
+    if (it == staged_.end() || it->second.shape.size() != 2 || it->second.shape[1] != cols) return -1;
+    return it->second.shape[0];
+  };
+  if (!up_mat("embed", vocab_, W, &embed_) || !up_mat("head", vocab_, W, &head_)) return false;
+  if (block_ == 2) {
+    if (!up_norm_off("final.norm", W, &final_norm_)) return false;
+    if (embed_norm_ && !up_norm_off("embed.norm", W, &embed_norm_w_)) return false;
+    if (pair_buckets_ > 0 && !up_mat("bigram", (int64_t)pair_buckets_ + 1, W, &pair_table_)) return false;
+  } else if (!up_norm("final.norm", &final_norm_, &final_b_, &final_alpha_)) {
+    return false;
+  }
   for (size_t li = 0; li < layers_.size(); li++) {
     StackLayer& L = layers_[li];
     if (L.weights_of >= 0) continue;
     const std::string p = "l" + std::to_string(li) + ".";
-    if (!up_norm(p + "norm1", &L.norm_w, &L.norm_b, &L.norm_alpha)) return false;
-    if (block_ == 1 && L.mlp != 0 && !up_norm(p + "norm2", &L.norm2_w, &L.norm2_b, &L.norm2_alpha)) return false;
-    if (L.mixer == 0) {  // q (| k | v) in one matrix: one launch projects them all
+    if (block_ == 2) {
+      if (!up_norm_off(p + "norm1", W, &L.norm_w) || !up_norm_off(p + "norm1b", W, &L.post1_w)) return false;
+      if (L.mlp != 0 && (!up_norm_off(p + "norm2", W, &L.norm2_w) || !up_norm_off(p + "norm2b", W, &L.post2_w))) return false;
+    } else {
+      if (!up_norm(p + "norm1", &L.norm_w, &L.norm_b, &L.norm_alpha)) return false;
+      if (block_ == 1 && L.mlp != 0 && !up_norm(p + "norm2", &L.norm2_w, &L.norm2_b, &L.norm2_alpha)) return false;
+    }
+    // two low-rank second stages side by side: [na + nb, ra + rb] with zeros off the diagonal blocks, so that one product serves both
+    auto block_diag = [&](const HostTensor* a2, int na, int ra, const HostTensor* b2, int nb, int rb, void** dst) {
+      const int R = ra + rb;
+      std::vector<uint8_t> m((size_t)(na + nb) * R * es, 0);
+      for (int r = 0; r < na; r++) memcpy(m.data() + (size_t)r * R * es, a2->data.data() + (size_t)r * ra * es, (size_t)ra * es);
+      for (int r = 0; r < nb; r++) memcpy(m.data() + ((size_t)(na + r) * R + ra) * es, b2->data.data() + (size_t)r * rb * es, (size_t)rb * es);
+      weight_bytes_ += m.size();
+      return (*dst = upload(m.data(), m.size())) != nullptr;
+    };
+    if (L.mixer == 3) {
+      // gated delta rule: q | k | v | write strengths in one matrix; the first stages of the decay and gate projections in a second one,
+      // their second stages block-diagonal in a third
+      const int H = L.heads, nk = L.nk(), nv = H * L.vdim, C = L.conv_channels();
+      const int64_t ra = rows_of(p + "mix.a1", W), rg = rows_of(p + "mix.g1", W);
+      if (ra < 1 || rg < 1) return error = "tensor " + p + "mix.a1 / g1: missing or of another width", false;
+      L.rank_a = (int)ra, L.rank_g = (int)rg;
+      const HostTensor *q, *k, *v, *bw, *a1, *g1, *a2, *g2, *cq, *ck, *cv, *al;
+      if (!need(p + "mix.q", nk, W, &q) || !need(p + "mix.k", nk, W, &k) || !need(p + "mix.v", nv, W, &v) || !need(p + "mix.b", H, W, &bw) ||
+          !need(p + "mix.a1", ra, W, &a1) || !need(p + "mix.g1", rg, W, &g1) || !need(p + "mix.a2", (int64_t)H * L.dim, ra, &a2) ||
+          !need(p + "mix.g2", nv, rg, &g2) || !matrix(q) || !matrix(k) || !matrix(v) || !matrix(bw) || !matrix(a1) || !matrix(g1) || !matrix(a2) || !matrix(g2))
+        return false;
+      if (!up_rows({q, k, v, bw}, &L.qkv) || !up_rows({a1, g1}, &L.lr1) || !block_diag(a2, H * L.dim, (int)ra, g2, nv, (int)rg, &L.lr2)) return false;
+      if (!need(p + "mix.q.conv", nk, L.conv, &cq) || !need(p + "mix.k.conv", nk, L.conv, &ck) || !need(p + "mix.v.conv", nv, L.conv, &cv)) return false;
+      std::vector<float> cw;
+      f32_of(*cq, &cw), f32_of(*ck, &cw), f32_of(*cv, &cw);
+      if ((int)cw.size() != C * L.conv || !(L.conv_w = upload_floats(cw))) return false;
+      if (!need(p + "mix.A_log", H, -1, &al)) return false;
+      std::vector<float> rate;
+      f32_of(*al, &rate);
+      for (float& r : rate) r = expf(r);
+      if (!(L.rate = upload_floats(rate)) || !up_vec(p + "mix.dt_bias", (int64_t)H * L.dim, &L.dt_bias) || !up_vec(p + "mix.norm", L.vdim, &L.out_norm_w)) return false;
+      if (!up_mat(p + "mix.o", W, nv, &L.o)) return false;
+    } else if (L.mixer == 4) {
+      const int H = L.heads;
+      const HostTensor *q, *k, *v, *g;
+      if (!need(p + "mix.q", (int64_t)H * L.dim, W, &q) || !need(p + "mix.k", (int64_t)H * L.dim, W, &k) || !need(p + "mix.v", (int64_t)H * L.vdim, W, &v) ||
+          !need(p + "mix.g", (int64_t)H * L.vdim, W, &g) || !matrix(q) || !matrix(k) || !matrix(v) || !matrix(g))
+        return false;
+      if (!up_rows({q, k, v, g}, &L.qkv) || !(L.head_decay = upload_floats(L.decay)) || !up_mat(p + "mix.o", W, H * L.vdim, &L.o)) return false;
+      rotary_table(L);
+      if (!L.freq_hi || !L.freq_lo) return false;
+    } else if (L.mixer == 5) {
+      const std::string pl = p + "mix.left.", pr = p + "mix.right.";
+      const int rq = L.r_heads * L.r_dim, rv = L.r_heads * L.r_vdim;
+      const int64_t ra = rows_of(pr + "a1", W);
+      if (ra < 1) return error = "tensor " + pr + "a1: missing or of another width", false;
+      L.rank_a = (int)ra;
+      const HostTensor *q, *k, *v, *q2, *k2, *v2, *g2, *a1;
+      if (!need(pl + "q", L.nq(), W, &q) || !need(pl + "k", L.nk(), W, &k) || !need(pl + "v", L.nv(), W, &v) || !need(pr + "q", rq, W, &q2) ||
+          !need(pr + "k", rq, W, &k2) || !need(pr + "v", rv, W, &v2) || !need(pr + "g", rv, W, &g2) || !need(pr + "a1", ra, W, &a1) || !matrix(q) || !matrix(k) ||
+          !matrix(v) || !matrix(q2) || !matrix(k2) || !matrix(v2) || !matrix(g2) || !matrix(a1))
+        return false;
+      if (!up_rows({q, k, v, q2, k2, v2, g2}, &L.qkv) || !up_rows({a1}, &L.lr1)) return false;
+      std::vector<float> bias;
+      if (L.has_bias) {
+        const HostTensor *qb, *kb, *vb;
+        if (!need(pl + "q.b", L.nq(), -1, &qb) || !need(pl + "k.b", L.nk(), -1, &kb) || !need(pl + "v.b", L.nv(), -1, &vb)) return false;
+        f32_of(*qb, &bias), f32_of(*kb, &bias), f32_of(*vb, &bias);
+        bias.resize(L.nqkv(), 0.f);
+        if (!(L.qkv_bias = upload_floats(bias))) return false;
+      }
+      if (L.qk_norm && (!up_vec(pl + "q.norm", L.dim, &L.qn_w) || !up_vec(pl + "k.norm", L.dim, &L.kn_w))) return false;
+      if (!up_mat(pl + "o", W, L.heads * L.vdim, &L.o) || !up_mat(pr + "o", W, rv, &L.r_o) || !up_mat(pr + "a2", rq, ra, &L.lr2) ||
+          !up_vec(pr + "a2.b", rq, &L.lr2_bias) || !up_vec(pr + "norm", L.r_vdim, &L.out_norm_w))
+        return false;
+      rotary_table(L);
+      if (!L.freq_hi || !L.freq_lo) return false;
+    } else if (L.mixer == 0) {  // q (| k | v) in one matrix: one launch projects them all
       const HostTensor *q, *k = nullptr, *v = nullptr;
       if (!need(p + "mix.q", L.nq(), W, &q) || !matrix(q)) return false;
       if (L.owns_cache && (!need(p + "mix.k", L.nk(), W, &k) || !need(p + "mix.v", L.nv(), W, &v) || !matrix(k) || !matrix(v))) return false;
@@ -347,7 +472,7 @@ bool StackModel::finalize_weights() {
         if (!(L.slopes = upload_floats(sl))) return false;
       }
     }
-    if (!up_mat(p + "mix.o", W, L.heads * L.vdim, &L.o)) return false;
+    if (L.mixer < 3 && !up_mat(p + "mix.o", W, L.heads * L.vdim, &L.o)) return false;
     if (L.mlp == 1) {
       if (!up_mat(p + "mlp.up", L.ff, W, &L.up) || !up_mat(p + "mlp.down", W, L.ff, &L.down) || !up_vec(p + "mlp.act", 4, &L.act)) return false;
     } else if (L.mlp == 3) {
@@ -367,6 +492,7 @@ bool StackModel::finalize_weights() {
       if (sg) rt.insert(rt.end(), sg->data.begin(), sg->data.end());
       weight_bytes_ += rt.size();
       if (!(L.router = upload(rt.data(), rt.size()))) return false;
+      if (L.router_kind == 1 && !up_vec(p + "mlp.router.b", L.experts, &L.router_bias)) return false;
       std::vector<uint8_t> gu((size_t)L.experts * 2 * L.ffp * W * es), dn((size_t)L.experts * W * L.ffp * es);
       for (int e = 0; e < L.experts; e++) {
         const std::string pe = p + "mlp.e" + std::to_string(e) + ".";
@@ -442,15 +568,48 @@ bool StackModel::init_synthetic(uint64_t seed) {
     put(name, W, 0, 1, 0.05);
     if (norm_kind_ == 1) put(name + ".b", W, 0, 0, 0.02), put(name + ".alpha", 1, 0, 0.5, 0.0);
   };
-  put_norm("final.norm");
+  if (block_ == 2) {  // norm weights are stored around zero; the embedding's own norm and the token-pair table
+    put("final.norm", W, 0, 0, 0.05);
+    if (embed_norm_) put("embed.norm", W, 0, 0, 0.05);
+    if (pair_buckets_ > 0) put("bigram", (int64_t)pair_buckets_ + 1, W, 0, 1.0);
+  } else {
+    put_norm("final.norm");
+  }
   for (size_t li = 0; li < layers_.size(); li++) {
     const StackLayer& L = layers_[li];
     if (L.weights_of >= 0) continue;
     const std::string p = "l" + std::to_string(li) + ".";
     const double sw = 1.0 / sqrt((double)W);
-    put_norm(p + "norm1");
-    if (block_ == 1 && L.mlp != 0) put_norm(p + "norm2");
-    if (L.mixer == 0) {
+    if (block_ == 2) {
+      put(p + "norm1", W, 0, 0, 0.05), put(p + "norm1b", W, 0, 0, 0.05);
+      if (L.mlp != 0) put(p + "norm2", W, 0, 0, 0.05), put(p + "norm2b", W, 0, 0, 0.05);
+    } else {
+      put_norm(p + "norm1");
+      if (block_ == 1 && L.mlp != 0) put_norm(p + "norm2");
+    }
+    if (L.mixer == 3) {
+      const int H = L.heads, nk = L.nk(), nv = H * L.vdim;
+      put(p + "mix.q", nk, W, 0, sw), put(p + "mix.k", nk, W, 0, sw), put(p + "mix.v", nv, W, 0, sw), put(p + "mix.b", H, W, 0, sw);
+      put(p + "mix.q.conv", nk, L.conv, 0.3, 0.3), put(p + "mix.k.conv", nk, L.conv, 0.3, 0.3), put(p + "mix.v.conv", nv, L.conv, 0.3, 0.3);
+      put(p + "mix.a1", L.rank_a, W, 0, sw), put(p + "mix.a2", (int64_t)H * L.dim, L.rank_a, 0, 1.0 / sqrt((double)L.rank_a));
+      put(p + "mix.g1", L.rank_g, W, 0, sw), put(p + "mix.g2", nv, L.rank_g, 0, 1.0 / sqrt((double)L.rank_g));
+      put(p + "mix.A_log", H, 0, -1.0, 0.5), put(p + "mix.dt_bias", (int64_t)H * L.dim, 0, -2.0, 1.0), put(p + "mix.norm", L.vdim, 0, 1, 0.05);
+      put(p + "mix.o", W, nv, 0, 1.0 / sqrt((double)nv));
+    } else if (L.mixer == 4) {
+      const int H = L.heads;
+      put(p + "mix.q", (int64_t)H * L.dim, W, 0, sw), put(p + "mix.k", (int64_t)H * L.dim, W, 0, sw), put(p + "mix.v", (int64_t)H * L.vdim, W, 0, sw);
+      put(p + "mix.g", (int64_t)H * L.vdim, W, 0, sw), put(p + "mix.o", W, H * L.vdim, 0, 1.0 / sqrt((double)H * L.vdim));
+    } else if (L.mixer == 5) {
+      const std::string pl = p + "mix.left.", pr = p + "mix.right.";
+      const int rq = L.r_heads * L.r_dim, rv = L.r_heads * L.r_vdim;
+      put(pl + "q", L.nq(), W, 0, sw), put(pl + "k", L.nk(), W, 0, sw), put(pl + "v", L.nv(), W, 0, sw);
+      if (L.has_bias) put(pl + "q.b", L.nq(), 0, 0, 0.02), put(pl + "k.b", L.nk(), 0, 0, 0.02), put(pl + "v.b", L.nv(), 0, 0, 0.02);
+      if (L.qk_norm) put(pl + "q.norm", L.dim, 0, 1, 0.05), put(pl + "k.norm", L.dim, 0, 1, 0.05);
+      put(pl + "o", W, L.heads * L.vdim, 0, 1.0 / sqrt((double)L.heads * L.vdim));
+      put(pr + "q", rq, W, 0, sw), put(pr + "k", rq, W, 0, sw), put(pr + "v", rv, W, 0, sw), put(pr + "g", rv, W, 0, sw);
+      put(pr + "a1", L.rank_a, W, 0, sw), put(pr + "a2", rq, L.rank_a, 0, 1.0 / sqrt((double)L.rank_a)), put(pr + "a2.b", rq, 0, 2.0, 1.0);
+      put(pr + "norm", L.r_vdim, 0, 1, 0.05), put(pr + "o", W, rv, 0, 1.0 / sqrt((double)rv));
+    } else if (L.mixer == 0) {
       put(p + "mix.q", L.nq(), W, 0, sw);
       if (L.owns_cache) put(p + "mix.k", L.nk(), W, 0, sw), put(p + "mix.v", L.nv(), W, 0, sw);
     } else if (L.mixer == 1) {
@@ -467,7 +626,7 @@ bool StackModel::init_synthetic(uint64_t seed) {
       put(p + "mix.q.norm", L.nq(), 0, 1, 0.05), put(p + "mix.k.norm", L.nk(), 0, 1, 0.05);
       put(p + "mix.pb", L.heads, 0, -3.0, 0.5), put(p + "mix.talk", L.heads, L.heads, 1.0 / L.heads, 0.1 / L.heads);
     }
-    put(p + "mix.o", W, L.heads * L.vdim, 0, 1.0 / sqrt((double)L.heads * L.vdim));
+    if (L.mixer < 3) put(p + "mix.o", W, L.heads * L.vdim, 0, 1.0 / sqrt((double)L.heads * L.vdim));
     if (L.mlp == 3) {
       put(p + "mlp.gate", L.ff, W, 0, sw), put(p + "mlp.up", L.ff, W, 0, sw), put(p + "mlp.down", W, L.ff, 0, 1.0 / sqrt((double)L.ff));
     } else if (L.mlp == 1) {
@@ -479,6 +638,7 @@ bool StackModel::init_synthetic(uint64_t seed) {
       staged_[p + "mlp.act"] = a;
     } else if (L.mlp == 2) {
       put(p + "mlp.router", L.experts, W, 0, sw);
+      if (L.router_kind == 1) put(p + "mlp.router.b", L.experts, 0, 0, 0.1);
       for (int e = 0; e < L.experts; e++) {
         const std::string pe = p + "mlp.e" + std::to_string(e) + ".";
         put(pe + "gate", L.ff, W, 0, sw), put(pe + "up", L.ff, W, 0, sw), put(pe + "down", W, L.ff, 0, 1.0 / sqrt((double)L.ff));
@@ -506,7 +666,7 @@ size_t StackModel::v_block_bytes(int c) const {
 int64_t StackModel::kv_bytes_per_block() const {
   int64_t b = 0;
   for (size_t c = 0; c < cache_layer_.size(); c++) b += (int64_t)k_block_bytes((int)c) + (int64_t)v_block_bytes((int)c);
-  return b;
+  return std::max<int64_t>(b, 16);  // (a stack without any cached layer still plans a block count)
 }
 bool StackModel::init_kv_cache(int num_blocks) {
   if (!spec_error_.empty()) return error = spec_error_, false;
@@ -521,20 +681,76 @@ bool StackModel::init_kv_cache(int num_blocks) {
   return hipDeviceSynchronize() == hipSuccess;
 }
 
+// what one sequence carries between steps: per recurrent layer the matrix state of every head (f32) and the last inputs of its short
+// convolutions
+int64_t StackModel::state_bytes_per_slot() const {
+  int64_t b = 0;
+  for (const StackLayer& L : layers_) {
+    if (L.s_heads() <= 0) continue;
+    b += (int64_t)L.s_heads() * L.s_dim() * L.s_vdim() * 4;
+    if (L.conv > 1) b += (int64_t)(L.conv - 1) * L.conv_channels() * 4;
+  }
+  return b;
+}
+bool StackModel::init_state(int slots) {
+  if (!spec_error_.empty()) return error = spec_error_, false;
+  state_slots_ = slots;
+  for (StackLayer& L : layers_) {
+    if (L.s_heads() <= 0) continue;
+    const size_t sb = (size_t)slots * L.s_heads() * L.s_dim() * L.s_vdim() * 4;
+    if (!(L.state = (float*)dalloc(sb)) || hipMemset(L.state, 0, sb) != hipSuccess) return error = "state slots: allocation failed", false;
+    if (L.conv > 1) {
+      const size_t cb = (size_t)slots * (L.conv - 1) * L.conv_channels() * 4;
+      if (!(L.conv_state = (float*)dalloc(cb)) || hipMemset(L.conv_state, 0, cb) != hipSuccess) return error = "state slots: allocation failed", false;
+    }
+  }
+  return hipDeviceSynchronize() == hipSuccess;
+}
+
+// rotary frequencies base^(-2i / dims) in f64, optionally slowed down by wavelength (waves longer than original / low are divided by
+// `factor`, shorter than original / high kept, those between blended linearly in original / wavelength), kept as hi + lo f32 pairs
+void StackModel::rotary_table(StackLayer& L) {
+  L.rot_pairs = L.rot_dims / 2;
+  L.rot_mag = 1.f;
+  std::vector<float> fh(std::max(L.rot_pairs, 1), 0.f), fl(std::max(L.rot_pairs, 1), 0.f);
+  for (int i = 0; i < L.rot_pairs; i++) {
+    double fr = pow(L.rot_base, -2.0 * (double)i / (double)L.rot_dims);
+    if (L.rs_factor > 0.0) {
+      const double wl = 2.0 * M_PI / fr;
+      if (wl > L.rs_original / L.rs_low) fr = fr / L.rs_factor;
+      else if (!(wl < L.rs_original / L.rs_high)) {
+        const double sm = (L.rs_original / wl - L.rs_low) / (L.rs_high - L.rs_low);
+        fr = (1.0 - sm) * fr / L.rs_factor + sm * fr;
+      }
+    }
+    fh[i] = (float)fr, fl[i] = (float)(fr - (double)fh[i]);
+  }
+  L.freq_hi = upload_floats(fh), L.freq_lo = upload_floats(fl);
+}
+
 bool StackModel::init_buffers(int max_tokens, int max_seqs) {
   if (!spec_error_.empty()) return error = spec_error_, false;
   max_tokens_ = max_tokens, max_seqs_ = max_seqs;
   const size_t T = max_tokens, W = width_;
   size_t nqkv = 0, nattn = 0, zc = 0, actc = 0, top = 0, experts = 0;
-  size_t nqa = 0;
+  size_t nqa = 0, z2c = 0, recc = 0, roc = 0;
   for (const StackLayer& L : layers_) {
     // softmax / sigmoid: the joint projection in the model's type; latent: q, later the heads' values (the joint projection is f32 in z_)
     nqkv = std::max(nqkv, L.mixer == 0 ? (size_t)L.nqkv() : std::max((size_t)L.nq(), (size_t)L.heads * L.vdim));
+    if (L.mixer >= 3) zc = std::max(zc, T * L.nqkv());
     nattn = std::max(nattn, (size_t)L.heads * (L.mixer == 1 ? L.kv_rank : L.vdim));
     if (L.mixer == 1) nqa = std::max(nqa, (size_t)L.heads * (L.kv_rank + L.rot_dim)), actc = std::max(actc, T * L.q_rank);
     if (L.mixer != 0) zc = std::max(zc, T * L.nqkv());
     if (L.mlp == 2) top = std::max(top, (size_t)L.top), experts = std::max(experts, (size_t)L.experts);
     if (L.mlp == 3) zc = std::max(zc, T * 2 * L.sffp), actc = std::max(actc, T * L.sffp);
+    if (L.mixer >= 3) {  // the joint projection is f32 in z_, the low-rank first stages in act_, their second stages in z2_
+      const size_t sh = L.s_heads(), sd = L.s_dim(), sv = L.s_vdim();
+      nattn = std::max(nattn, sh * sv);
+      actc = std::max(actc, T * (size_t)(L.rank_a + L.rank_g));
+      z2c = std::max(z2c, sh * sd + (L.mixer == 3 ? sh * sv : 0));
+      recc = std::max(recc, L.mixer == 3 ? (size_t)L.conv_channels() + sh + sh * sd : (L.mixer == 4 ? 2 * sh * sd : sh * sd));
+      roc = std::max(roc, sh * sv);
+    }
   }
   max_rows_ = (int)round_up((int)(T * std::max<size_t>(top, 1) + experts * 63), 64);
   for (const StackLayer& L : layers_) {
@@ -552,6 +768,7 @@ bool StackModel::init_buffers(int max_tokens, int max_seqs) {
       !(pair_out_ = (float*)dalloc(T * std::max<size_t>(top, 1) * W * 4)) || !(sh_ = (float*)dalloc(T * W * 4)) || !(xl_ = (float*)dalloc(R * W * 4)) ||
       !(hl_ = dalloc(R * W * es_)) || !(logits_ = (float*)dalloc(R * (size_t)vocab_ * 4)) || !(qa_ = dalloc(std::max<size_t>(T * nqa, 4) * es_)))
     return false;
+  if (z2c && (!(z2_ = (float*)dalloc(T * z2c * 4)) || !(rec_ = (float*)dalloc(T * recc * 4)) || !(ro_ = (float*)dalloc(T * roc * 4)))) return false;
   // sigmoid attention sums in two launches: per-head-pair sums of a prompt portion (bf16, at most 1 GiB: longer steps take the one-launch
   // kernel), per-tile partial sums of decoded tokens
   for (const StackLayer& L : layers_) {
@@ -757,11 +974,15 @@ bool StackModel::forward(const InputMetadata& md, int64_t stream, uint32_t* toke
     }
     trace_bytes_ = need_b;
   }
-  vra_stack_embed_sinpos(md.input_ids, md.positions, embed_, pos_kind_ == 0 ? inv_freq_ : nullptr, x_, T, W, vocab_, dt_, stream);
-  if (take_stack_err(error, "embedding")) return false;
+  if (block_ == 2) {
+    if (!forward_sandwich(md, stream)) return false;
+  } else {
+    vra_stack_embed_sinpos(md.input_ids, md.positions, embed_, pos_kind_ == 0 ? inv_freq_ : nullptr, x_, T, W, vocab_, dt_, stream);
+    if (take_stack_err(error, "embedding")) return false;
+  }
   // sequential blocks: the output of a sub-block is added to the residual inside the launch of the next norm (`pending`)
   const float* pending = nullptr;
-  for (size_t li = 0; li < layers_.size(); li++) {
+  for (size_t li = 0; li < layers_.size() && block_ != 2; li++) {
     const StackLayer& L = layers_[li];
     if (block_ == 0) {
       // h = norm(x); a mixture-of-experts layer's router (and its shared expert's gate) reads h inside the same launch
@@ -817,6 +1038,174 @@ bool StackModel::forward(const InputMetadata& md, int64_t stream, uint32_t* toke
   vra_stack_gemm(hd, dt_, stream);
   if (tokens) vra_argmax_f32(logits_, tokens, rows, vocab_, stream);
   return !take_stack_err(error, "head");
+}
+
+// ---------------------------------------------------------------------------------------------
+// sandwich blocks with recurrent mixers
+// ---------------------------------------------------------------------------------------------
+// the recurrence has left o (f32 [T, heads * vdim]) in ro_: per-head norm, gate, output projection -> out (f32 [T, width])
+bool StackModel::recurrent_tail(const StackLayer& L, const InputMetadata& md, const float* gate, int gate_ld, int gate_act, const void* w_o, float* out,
+                                int64_t stream) {
+  const int T = md.n_tokens, H = L.s_heads(), V = L.s_vdim();
+  vra_stack_head_norm_gate(ro_, L.out_norm_w, gate, gate_ld, gate_act, eps_, attn_, T, H, V, dt_, stream);
+  StkGemmArgs o;
+  o.a = attn_, o.lda = H * V, o.w = w_o, o.M = T, o.N = width_, o.K = H * V, o.out = out, o.ldo = width_, o.out_f32 = 1;
+  vra_stack_gemm(o, dt_, stream);
+  return !take_stack_err(error, "recurrent mixer");
+}
+
+static void scan_common(StkScanArgs& sc, const StackLayer& L, const InputMetadata& md, float* out) {
+  sc.state = L.state, sc.state_slots = md.state_slots, sc.positions = md.positions, sc.cu_q = md.is_prefill ? md.cu_seqlens_q : nullptr;
+  sc.out = out, sc.ldo = L.s_heads() * L.s_vdim(), sc.B = md.n_seqs, sc.H = L.s_heads(), sc.dim = L.s_dim(), sc.vdim = L.s_vdim();
+}
+
+// gated delta rule: joint projection (f32), the low-rank first stages (model type) and their second stages (f32), then one launch for
+// the convolutions, unit vectors, write strengths and decays, one that moves the convolution state on, the recurrence, norm + gate, o
+bool StackModel::mixer_delta(const StackLayer& L, const InputMetadata& md, int64_t stream) {
+  const int T = md.n_tokens, W = width_, H = L.heads, G = L.kv_heads, D = L.dim, V = L.vdim, n1 = L.nqkv(), C = L.conv_channels(), R = L.rank_a + L.rank_g;
+  StkGemmArgs p;
+  p.a = h_, p.lda = W, p.w = L.qkv, p.M = T, p.N = n1, p.K = W, p.out = z_, p.ldo = n1, p.out_f32 = 1;
+  vra_stack_gemm(p, dt_, stream);
+  StkGemmArgs l1;
+  l1.a = h_, l1.lda = W, l1.w = L.lr1, l1.M = T, l1.N = R, l1.K = W, l1.out = act_, l1.ldo = R;
+  vra_stack_gemm(l1, dt_, stream);
+  const int n2 = H * D + H * V;
+  StkGemmArgs l2;
+  l2.a = act_, l2.lda = R, l2.w = L.lr2, l2.M = T, l2.N = n2, l2.K = R, l2.out = z2_, l2.ldo = n2, l2.out_f32 = 1;
+  vra_stack_gemm(l2, dt_, stream);
+  StkDeltaPrepArgs d;
+  d.raw = z_, d.ld = n1, d.raw2 = z2_, d.ld2 = n2, d.conv_w = L.conv_w, d.taps = L.conv, d.conv_state = L.conv_state ? L.conv_state : z2_;
+  d.rate = L.rate, d.dt_bias = L.dt_bias, d.q_scale = 1.f / sqrtf((float)D);
+  d.qkv_out = rec_, d.beta_out = rec_ + (size_t)T * C, d.decay_out = rec_ + (size_t)T * (C + H);
+  d.positions = md.positions, d.cu_q = md.is_prefill ? md.cu_seqlens_q : nullptr, d.state_slots = md.state_slots;
+  d.T = T, d.B = md.n_seqs, d.H = H, d.G = G, d.dim = D, d.vdim = V;
+  vra_stack_delta_prep(d, stream);
+  vra_stack_conv_state_update(d, stream);
+  StkScanArgs sc;
+  sc.q = rec_, sc.ldq = C, sc.k = rec_ + G * D, sc.ldk = C, sc.v = rec_ + 2 * G * D, sc.ldv = C, sc.qk_rep = H / G;
+  sc.decay = d.decay_out, sc.ldd = H * D, sc.beta = d.beta_out, sc.ldb = H;
+  scan_common(sc, L, md, ro_);
+  vra_stack_linear_scan(sc, stream);
+  if (take_stack_err(error, "delta rule")) return false;
+  return recurrent_tail(L, md, z2_ + H * D, n2, 2, L.o, o_, stream);
+}
+
+// retention: q | k | v | gate in one launch (f32), rotary on q and k with the key's scale, the recurrence with one decay per head
+bool StackModel::mixer_retention(const StackLayer& L, const InputMetadata& md, int64_t stream) {
+  const int T = md.n_tokens, W = width_, H = L.heads, D = L.dim, V = L.vdim, n1 = L.nqkv();
+  StkGemmArgs p;
+  p.a = h_, p.lda = W, p.w = L.qkv, p.M = T, p.N = n1, p.K = W, p.out = z_, p.ldo = n1, p.out_f32 = 1;
+  vra_stack_gemm(p, dt_, stream);
+  StkHeadPrepArgs hp;
+  hp.raw = z_, hp.ld = n1, hp.q_off = 0, hp.k_off = H * D, hp.Hq = H, hp.Hk = H, hp.dim = D, hp.eps = eps_;
+  hp.rot.freq_hi = L.freq_hi, hp.rot.freq_lo = L.freq_lo, hp.rot.pairs = L.rot_pairs, hp.rot.mag = 1.f;
+  hp.k_scale = 1.f / sqrtf((float)D), hp.positions = md.positions;
+  hp.q_out = rec_, hp.q_ld = 2 * H * D, hp.k_out = rec_ + H * D, hp.k_ld = 2 * H * D, hp.out_f32 = 1, hp.T = T;
+  vra_stack_head_prep(hp, dt_, stream);
+  StkScanArgs sc;
+  sc.q = rec_, sc.ldq = 2 * H * D, sc.k = rec_ + H * D, sc.ldk = 2 * H * D, sc.v = z_ + 2 * H * D, sc.ldv = n1, sc.head_decay = L.head_decay;
+  scan_common(sc, L, md, ro_);
+  vra_stack_linear_scan(sc, stream);
+  if (take_stack_err(error, "retention")) return false;
+  return recurrent_tail(L, md, z_ + 2 * H * D + H * V, n1, 1, L.o, o_, stream);
+}
+
+// two branches on one input.  Left: softmax attention over the paged cache (biases in the projection's epilogue, per-head q / k norm and
+// rotary in the launch that writes the cache rows, visibility inside blocks of `chunk` positions) -> o_.  Right: gated linear attention
+// (decay per key channel sigmoid(z)^(1 / tau), z from a low-rank projection with a bias) -> sh_.  The caller sums them with their scales.
+bool StackModel::mixer_parallel(const StackLayer& L, const InputMetadata& md, int64_t stream) {
+  const int T = md.n_tokens, B = md.n_seqs, W = width_, n1 = L.nqkv(), H = L.heads, RH = L.r_heads, RD = L.r_dim, RV = L.r_vdim;
+  const int lq = L.nq(), lk = L.nk(), lv = L.nv(), r0 = lq + lk + lv;
+  StkGemmArgs p;
+  p.a = h_, p.lda = W, p.w = L.qkv, p.bias = L.qkv_bias, p.M = T, p.N = n1, p.K = W, p.out = z_, p.ldo = n1, p.out_f32 = 1;
+  vra_stack_gemm(p, dt_, stream);
+  StkGemmArgs l1;
+  l1.a = h_, l1.lda = W, l1.w = L.lr1, l1.M = T, l1.N = L.rank_a, l1.K = W, l1.out = act_, l1.ldo = L.rank_a;
+  vra_stack_gemm(l1, dt_, stream);
+  StkGemmArgs l2;
+  l2.a = act_, l2.lda = L.rank_a, l2.w = L.lr2, l2.bias = L.lr2_bias, l2.M = T, l2.N = RH * RD, l2.K = L.rank_a, l2.out = z2_, l2.ldo = RH * RD, l2.out_f32 = 1;
+  vra_stack_gemm(l2, dt_, stream);
+  // left
+  StkHeadPrepArgs hp;
+  hp.raw = z_, hp.ld = n1, hp.q_off = 0, hp.k_off = lq, hp.v_off = lq + lk, hp.Hq = H, hp.Hk = L.kv_heads, hp.dim = L.dim, hp.nv = lv;
+  hp.qn_w = L.qn_w, hp.kn_w = L.kn_w, hp.eps = eps_;
+  hp.rot.freq_hi = L.freq_hi, hp.rot.freq_lo = L.freq_lo, hp.rot.pairs = L.rot_pairs, hp.rot.mag = 1.f;
+  hp.positions = md.positions, hp.q_out = qkv_, hp.q_ld = lq, hp.k_out = kc_[L.cache], hp.k_ld = lk, hp.v_out = vc_[L.cache], hp.v_ld = lv;
+  hp.slots = md.slot_mapping, hp.T = T;
+  vra_stack_head_prep(hp, dt_, stream);
+  StkAttnArgs a;
+  a.q = qkv_, a.ldq = lq, a.out = attn_, a.kc = kc_[L.cache], a.vc = vc_[L.cache];
+  a.positions = md.positions, a.block_tables = md.block_tables, a.context_lens = md.context_lens;
+  a.cu_q = md.is_prefill ? md.cu_seqlens_q : nullptr;
+  a.B = B, a.T = T, a.max_q = md.is_prefill ? md.max_seqlen_q : 1, a.H = H, a.G = L.kv_heads, a.dim = L.dim, a.vdim = L.vdim;
+  a.BS = ec_.block_size, a.max_blocks = md.max_blocks, a.scale = L.scale, a.chunk = L.chunk;
+  vra_stack_attention(a, dt_, stream);
+  StkGemmArgs o;
+  o.a = attn_, o.lda = H * L.vdim, o.w = L.o, o.M = T, o.N = W, o.K = H * L.vdim, o.out = o_, o.ldo = W, o.out_f32 = 1;
+  vra_stack_gemm(o, dt_, stream);
+  if (take_stack_err(error, "parallel mixer (attention)")) return false;
+  // right
+  vra_stack_sigmoid_pow(z2_, RH * RD, rec_, RH * RD, T, RH * RD, 1.f / L.tau, stream);
+  StkScanArgs sc;
+  sc.q = z_ + r0, sc.ldq = n1, sc.k = z_ + r0 + RH * RD, sc.ldk = n1, sc.v = z_ + r0 + 2 * RH * RD, sc.ldv = n1, sc.q_scale = 1.f / sqrtf((float)RD);
+  sc.decay = rec_, sc.ldd = RH * RD;
+  scan_common(sc, L, md, ro_);
+  vra_stack_linear_scan(sc, stream);
+  if (take_stack_err(error, "parallel mixer (linear attention)")) return false;
+  return recurrent_tail(L, md, z_ + r0 + 2 * RH * RD + RH * RV, n1, 1, L.r_o, sh_, stream);
+}
+
+// embedding (+ token-pair table, + its norm), then per layer  x += N(mixer(N(x))),  x += N(ff(N(x))).  A sub-block's output is normed and
+// added inside the launch that norms the next sub-block's input (and, before a mixture of experts, runs its router).
+bool StackModel::forward_sandwich(const InputMetadata& md, int64_t stream) {
+  const int T = md.n_tokens, W = width_;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (!md.state_slots || !md.prev_tokens) return error = "forward: this model needs the sequences' state slots and previous tokens", false;
+  StkEmbedPairArgs e;
+  e.ids = md.input_ids, e.positions = md.positions, e.cu_q = md.is_prefill ? md.cu_seqlens_q : nullptr, e.prev_tokens = md.prev_tokens;
+  e.embed = embed_, e.table = pair_table_, e.buckets = pair_buckets_, e.mul_prev = pair_mul_prev_, e.mul_cur = pair_mul_cur_, e.scale = embed_scale_;
+  e.norm_w = embed_norm_w_, e.eps = eps_, e.x = x_, e.T = T, e.B = md.n_seqs, e.W = W, e.V = vocab_;
+  vra_stack_embed_pair(e, dt_, stream);
+  if (take_stack_err(error, "embedding")) return false;
+  StkSandwichArgs pend;  // the parts of the last sub-block's output, not yet normed and added (post_w null: none)
+  auto seam = [&](const float* pre_w, const StackLayer* router) {
+    StkSandwichArgs s = pend;
+    s.x = x_, s.pre_w = pre_w, s.h = h_, s.eps = eps_, s.T = T, s.W = W;
+    if (router) {
+      s.router_w = router->router, s.router_bias = router->router_bias, s.n_router = router->experts, s.top = router->top;
+      s.pair_expert = pair_expert_, s.pair_weight = pair_weight_;
+    }
+    if (s.post_w || s.pre_w) vra_stack_sandwich_norm(s, dt_, stream);
+    pend = StkSandwichArgs();
+    return !take_stack_err(error, "norm");
+  };
+  for (size_t li = 0; li < layers_.size(); li++) {
+    const StackLayer& L = layers_[li];
+    if (!seam(L.norm_w, nullptr)) return false;
+    if (!(L.mixer == 3 ? mixer_delta(L, md, stream) : (L.mixer == 4 ? mixer_retention(L, md, stream) : mixer_parallel(L, md, stream)))) return false;
+    pend.p1 = o_, pend.n1 = 1, pend.post_w = L.post1_w;
+    if (L.mixer == 5) pend.c1 = L.left_scale, pend.p2 = sh_, pend.c2 = L.right_scale;
+    if (L.mlp == 2) {
+      if (!seam(L.norm2_w, &L)) return false;
+      const int P = T * L.top;
+      const int granule = vra_stack_gemm_granule(P, L.experts);
+      const int rows = round_up(P + L.experts * (granule - 1), granule);
+      if (rows > max_rows_) return error = "feed-forward: more expert rows than the buffers hold", false;
+      vra_stack_moe_sort(pair_expert_, pair_weight_, P, L.top, L.experts, granule, rows, row_token_, row_scale_, row_pair_, tile_group_, stream);
+      if (take_stack_err(error, "expert rows")) return false;
+      // (the weights of a softmax router multiply the experts' OUTPUTS: the rows go in unscaled, the sum over a token's pairs carries them)
+      if (!expert_pair(h_, W, L.e_gu, (int64_t)2 * L.ffp * W, L.e_down, (int64_t)W * L.ffp, rows, L.ffp, L.ff, L.limit, tile_group_, granule, row_token_,
+                       L.router_kind == 1 ? nullptr : row_scale_, row_pair_, pair_out_, stream, L.act_kind))
+        return false;
+      pend.p1 = pair_out_, pend.n1 = L.top, pend.pw = L.router_kind == 1 ? pair_weight_ : nullptr, pend.post_w = L.post2_w;
+    }
+    if (trace_on_ || li + 1 == layers_.size()) {
+      if (!seam(nullptr, nullptr)) return false;
+      if (trace_on_ && hipMemcpyAsync(trace_ + li * (size_t)T * W, x_, (size_t)T * W * 4, hipMemcpyDeviceToDevice, st) != hipSuccess)
+        return error = "layer trace copy failed", false;
+    }
+  }
+  return true;
 }
 
 int64_t StackModel::read_layer_trace(void* host, int64_t max_bytes, int64_t stream) {

@@ -3,14 +3,24 @@
 //
 //   block   parallel:    x <- x + m * (mixer(h) + ff(h)),  h = norm(x)                      (Ditilix)
 //           sequential:  x <- x + mixer(norm1(x)),  x <- x + ff(norm2(x))                   (Gaperax)
+//           sandwich:    x <- x + norm1b(mixer(norm1(x))),  x <- x + norm2b(ff(norm2(x)))   (Zifetar; RMS norms, norm_offset added to the weights)
 //   norm    rms: RMS norm over `groups` equal parts of the width;  dyt: Dynamic Tanh  tanh(alpha x) w + b  (no statistics)
 //   pos     sinusoid: a position vector added to the embedding;  none: positions enter inside the mixers
+//   embedding (sandwich stacks): embed * embed_scale + a row of a hashed (previous token, token) table (pair_buckets, pair_mul_prev,
+//           pair_mul_cur; the table's last row for a sequence's first token), then an RMS norm of its own
 //   mixer   attention: causal softmax, query temperature, soft cap, grouped key/value heads, optionally another layer's keys / values
 //           latent:    queries and keys / values through low-rank latents, a rotated key part shared by the heads (rotary with optional
 //                      YaRN scaling), a softmax sink per head; the cache holds one row [latent | rotated part] per token and the
 //                      up-projections are absorbed: q' = [W_uk_h^T q_h | rot(q_h)], values = the latent, W_uv_h after the sum over keys
 //           sigmoid:   biased q / k / v, one RMS norm over all of q and all of k, weights sigmoid(score - slope_h * distance + bias_h)
 //                      without normalisation, a window that keeps the first tokens, heads mixed by a matrix, a sigmoid output gate
+//   delta:     gated delta rule: short causal convolutions + silu on q / k / v, unit-vector q and k, a write strength per head, a decay per
+//                      head and key channel from a low-rank projection, per-head output norm and a low-rank sigmoid gate
+//           retention: linear attention with a constant decay per head, rotary (rotate-half layout) on q and k, per-head output norm, silu gate
+//           parallel:  two branches on the same input, summed with constant scales: softmax attention (biases, per-head q / k norm, rotary
+//                      with wavelength-dependent scaling, visibility inside blocks of `chunk` positions) and a gated linear attention
+//                      (decay per key channel sigmoid(z)^(1 / tau) from a low-rank projection)
+//           delta, retention and the right branch keep a matrix state [dim, vdim] per head and sequence (f32, one slot per live sequence)
 //   mlp     none | dense (PolyNorm activation) | moe (sigmoid router, clamped gated experts, gated shared expert) | gated (gelu_tanh(gate) * up)
 //   weights_of=j: the layer runs with layer j's tensors and a cache of its own
 // vllm_rs_amd/checkpoint.py turns a design's config.json into the spec text below.
@@ -23,7 +33,9 @@
 //   layer mixer=.. heads=.. kv_heads=.. dim=.. vdim=.. scale=.. softcap=.. temp_coef=.. temp_every=.. kv_from=.. weights_of=..
 //         rot_dim=.. kv_rank=.. q_rank=.. rot_dims=.. rot_base=.. yarn_factor=.. yarn_original=.. yarn_fast=.. yarn_slow=.. sink=0|1
 //         window=.. keep_first=.. slope_exp=..
-//         mlp=none|dense|moe|gated ff=.. experts=.. top=.. limit=.. shared_ff=.. shared_limit=..
+//         conv=.. rank_a=.. rank_g=.. decay=d0,d1,.. chunk=.. qk_norm=0|1 bias=0|1 rs_factor=.. rs_low=.. rs_high=.. rs_original=..
+//         r_heads=.. r_dim=.. r_vdim=.. tau=.. left_scale=.. right_scale=..
+//         mlp=none|dense|moe|gated ff=.. experts=.. top=.. limit=.. shared_ff=.. shared_limit=.. router=sigmoid|softmax act=clamped|silu
 #pragma once
 #include <map>
 #include <string>
@@ -34,7 +46,8 @@
 namespace vra {
 
 struct StackLayer {
-  // mixer: 0 softmax attention, 1 latent attention, 2 sigmoid attention
+  // mixer: 0 softmax attention, 1 latent attention, 2 sigmoid attention, 3 gated delta rule, 4 retention, 5 parallel (softmax attention
+  // beside a gated linear attention)
   int mixer = 0;
   int heads = 0, kv_heads = 0, dim = 0, vdim = 0, temp_every = 0, kv_from = -1, weights_of = -1;
   float scale = 1.f, softcap = 0.f, temp_coef = 0.f;
@@ -44,9 +57,20 @@ struct StackLayer {
   // sigmoid attention: window <= 0 = every earlier token; slope_h = 2^(-slope_exp (h + 1) / heads), 0 = no distance penalty
   int window = 0, keep_first = 0;
   double slope_exp = 0.0;
+  // recurrent mixers.  delta: taps of the short convolutions, ranks of the decay / gate projections (a loaded checkpoint's tensor shapes
+  // override the ranks); retention: one decay per head; softmax branch of a parallel mixer: block mask, per-head q / k norm, biases,
+  // rotary scaling by wavelength (rs_factor 0: none); its right branch: r_* sizes, tau, and the two branches' scales
+  int conv = 0, rank_a = 0, rank_g = 0, chunk = 0, qk_norm = 0, has_bias = 0;
+  std::vector<float> decay;
+  double rs_factor = 0.0, rs_low = 1.0, rs_high = 4.0, rs_original = 0.0;
+  int r_heads = 0, r_dim = 0, r_vdim = 0;
+  float tau = 1.f, left_scale = 1.f, right_scale = 1.f;
   // feed-forward: 0 none, 1 dense (PolyNorm), 2 mixture of experts, 3 gated dense (gelu_tanh(gate) * up)
   int mlp = 0, ff = 0, experts = 0, top = 0, shared_ff = 0;
   float limit = 0.f, shared_limit = 0.f;
+  // mixture of experts: router 0 = sigmoid scores as weights on the experts' inputs, 1 = biased logits, softmax over the chosen ones, weights
+  // on the experts' outputs; act 0 = clamped gated form, 2 = silu(gate) * up
+  int router_kind = 0, act_kind = 0;
   // derived
   int cache = -1;          // index of the paged cache this layer reads (its own, or the one of layer kv_from)
   bool owns_cache = false;
@@ -58,8 +82,17 @@ struct StackLayer {
   int nqkv() const {
     if (mixer == 1) return q_rank + kv_rank + rot_dim;
     if (mixer == 2) return nq() + nk() + nv() + heads * vdim;
+    if (mixer == 3) return 2 * nk() + heads * vdim + heads;          // q | k (kv_heads each) | v | write strengths
+    if (mixer == 4) return 2 * heads * dim + 2 * heads * vdim;       // q | k | v | gate
+    if (mixer == 5) return nq() + nk() + nv() + r_heads * (2 * r_dim + 2 * r_vdim);  // left q | k | v, right q | k | v | gate
     return nq() + (owns_cache ? nk() + nv() : 0);
   }
+  bool has_cache() const { return mixer != 3 && mixer != 4; }
+  // the recurrent part: heads, key and value sizes of the matrix state (0 heads: none)
+  int s_heads() const { return mixer == 5 ? r_heads : (mixer == 3 || mixer == 4 ? heads : 0); }
+  int s_dim() const { return mixer == 5 ? r_dim : dim; }
+  int s_vdim() const { return mixer == 5 ? r_vdim : vdim; }
+  int conv_channels() const { return mixer == 3 ? 2 * nk() + heads * vdim : 0; }
   // elements of one token's cache rows
   int k_row() const { return mixer == 1 ? kv_rank + rot_dim : nk(); }
   int v_row() const { return mixer == 1 ? 0 : nv(); }
@@ -86,6 +119,16 @@ struct StackLayer {
   void* e_down = nullptr;  // [experts][width][ffp]
   void* s_gu = nullptr;    // [2 * sffp][width]  (shared expert, or the gated dense feed-forward)
   void* s_down = nullptr;  // [width][sffp]
+  // sandwich blocks and recurrent mixers
+  float *post1_w = nullptr, *post2_w = nullptr;  // norms of the mixer's / the feed-forward's output
+  float* router_bias = nullptr;
+  void* lr1 = nullptr;          // first stage of the low-rank projections [rank_a (+ rank_g), width]
+  void* lr2 = nullptr;          // second stage [heads * dim (+ heads * vdim), rank_a (+ rank_g)], block diagonal
+  float* lr2_bias = nullptr;
+  float *conv_w = nullptr, *rate = nullptr, *dt_bias = nullptr, *out_norm_w = nullptr, *head_decay = nullptr;
+  void* r_o = nullptr;          // right branch: [width, r_heads * r_vdim]
+  float* state = nullptr;       // [slots, heads, vdim, dim]
+  float* conv_state = nullptr;  // [slots, conv - 1, conv_channels()]
 };
 
 class StackModel : public ModelBase {
@@ -96,6 +139,8 @@ class StackModel : public ModelBase {
   bool load_tensor(const std::string& name, const void* host, const int64_t* shape, int ndim, int elem_bytes) override;
   bool finalize_weights() override;
   bool init_kv_cache(int num_blocks) override;
+  int64_t state_bytes_per_slot() const override;
+  bool init_state(int slots) override;
   int num_blocks() const override { return num_blocks_; }
   int kv_layers() const override { return (int)kc_.size(); }
   size_t k_block_bytes(int c) const override;
@@ -130,6 +175,12 @@ class StackModel : public ModelBase {
   bool mixer_softmax(const StackLayer& L, const InputMetadata& md, int64_t stream);
   bool mixer_latent(const StackLayer& L, const InputMetadata& md, int64_t stream);
   bool mixer_sigmoid(const StackLayer& L, const InputMetadata& md, int64_t stream);
+  bool mixer_delta(const StackLayer& L, const InputMetadata& md, int64_t stream);
+  bool mixer_retention(const StackLayer& L, const InputMetadata& md, int64_t stream);
+  bool mixer_parallel(const StackLayer& L, const InputMetadata& md, int64_t stream);
+  bool recurrent_tail(const StackLayer& L, const InputMetadata& md, const float* gate, int gate_ld, int gate_act, const void* w_o, float* out, int64_t stream);
+  bool forward_sandwich(const InputMetadata& md, int64_t stream);
+  void rotary_table(StackLayer& L);
   float* upload_floats(const std::vector<float>& v);
   bool norm_into_h(const float* w, const float* b, float alpha, const float* add, float* x, void* h, int T, int64_t stream);
   bool expert_pair(const void* a, int lda, const void* w_gu, int64_t gu_stride, const void* w_down, int64_t down_stride, int rows, int fp, int f,
@@ -141,7 +192,14 @@ class StackModel : public ModelBase {
   int dt_ = 0;
   size_t es_ = 2;
   int width_ = 0, vocab_ = 0, groups_ = 1;
-  int block_ = 0, norm_kind_ = 0, pos_kind_ = 0;  // 0 parallel / rms / sinusoid, 1 sequential / dyt / none
+  int block_ = 0, norm_kind_ = 0, pos_kind_ = 0;  // 0 parallel / rms / sinusoid, 1 sequential / dyt / none, block 2 sandwich
+  float norm_offset_ = 0.f, embed_scale_ = 1.f;    // added to every norm weight at load; multiplies the embedding row
+  int embed_norm_ = 0, pair_buckets_ = 0;
+  int64_t pair_mul_prev_ = 0, pair_mul_cur_ = 0;
+  void* pair_table_ = nullptr;
+  float* embed_norm_w_ = nullptr;
+  int state_slots_ = 0;
+  float *z2_ = nullptr, *rec_ = nullptr, *ro_ = nullptr;
   float eps_ = 1e-6f, residual_mult_ = 1.f, logit_scale_ = 1.f;
   double pos_base_ = 10000.0;
   std::vector<StackLayer> layers_;
