@@ -238,3 +238,73 @@ def forward(cfg, w, tokens, layers_out=None):
         if layers_out is not None:
             layers_out.append(x.copy())
     return norm1p(x, w["final.norm"], eps) @ w["head"].T
+
+
+def bf16_round(a):
+    """float32 array rounded to bfloat16 (nearest even), returned as float32"""
+    u = np.ascontiguousarray(a, np.float32).view(np.uint32).astype(np.uint64)
+    return (((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16).astype(np.uint32).view(np.float32).reshape(np.shape(a))
+
+
+def tensor_shapes(cfg, rank=8):
+    """name -> shape of every tensor a model of this config has; `rank` (or a mixer's "rank_a" / "rank_g") sizes the low-rank projections,
+    which a config does not carry"""
+    W, V = cfg["width"], cfg["vocab"]
+    out = {"embed": (V, W), "bigram": (cfg["embedding"]["bigram"]["buckets"] + 1, W), "embed.norm": (W,), "head": (V, W), "final.norm": (W,)}
+    for i, layer in enumerate(cfg["layers"]):
+        p = "l%d." % i
+        for n in ("norm1", "norm1b", "norm2", "norm2b") if layer.get("mlp") else ("norm1", "norm1b"):
+            out[p + n] = (W,)
+        mx, m = layer["mixer"], p + "mix."
+        if layer["type"] == "channel_delta":
+            H, G, D, Vd = mx["heads"], mx.get("kv_heads", mx["heads"]), mx["dim"], mx.get("vdim", mx["dim"])
+            ra, rg, taps = mx.get("rank_a", rank), mx.get("rank_g", rank), mx["conv"]
+            out.update({m + "q": (G * D, W), m + "q.conv": (G * D, taps), m + "k": (G * D, W), m + "k.conv": (G * D, taps), m + "v": (H * Vd, W),
+                        m + "v.conv": (H * Vd, taps), m + "b": (H, W), m + "A_log": (H,), m + "norm": (Vd,), m + "a1": (ra, W), m + "a2": (H * D, ra),
+                        m + "dt_bias": (H * D,), m + "g1": (rg, W), m + "g2": (H * Vd, rg), m + "o": (W, H * Vd)})
+        elif layer["type"] == "retention":
+            H, D, Vd = mx["heads"], mx["dim"], mx.get("vdim", mx["dim"])
+            out.update({m + "q": (H * D, W), m + "k": (H * D, W), m + "v": (H * Vd, W), m + "g": (H * Vd, W), m + "o": (W, H * Vd)})
+        else:
+            le, ri = mx["left"], mx["right"]
+            H, G, D, Vd = le["heads"], le.get("kv_heads", le["heads"]), le["dim"], le.get("vdim", le["dim"])
+            out.update({m + "left.q": (H * D, W), m + "left.q.b": (H * D,), m + "left.k": (G * D, W), m + "left.k.b": (G * D,), m + "left.v": (G * Vd, W),
+                        m + "left.v.b": (G * Vd,), m + "left.q.norm": (D,), m + "left.k.norm": (D,), m + "left.o": (W, H * Vd)})
+            H, D, Vd, ra = ri["heads"], ri["dim"], ri.get("vdim", ri["dim"]), ri.get("rank_a", rank)
+            out.update({m + "right.q": (H * D, W), m + "right.k": (H * D, W), m + "right.v": (H * Vd, W), m + "right.g": (H * Vd, W),
+                        m + "right.o": (W, H * Vd), m + "right.norm": (Vd,), m + "right.a1": (ra, W), m + "right.a2": (H * D, ra), m + "right.a2.b": (H * D,)})
+        if layer.get("mlp"):
+            f, E = layer["mlp"]["expert"]["ff"], layer["mlp"]["router"]["experts"]
+            out.update({p + "mlp.router": (E, W), p + "mlp.router.b": (E,)})
+            for e in range(E):
+                out.update({p + "mlp.e%d.gate" % e: (f, W), p + "mlp.e%d.up" % e: (f, W), p + "mlp.e%d.down" % e: (W, f)})
+    return out
+
+
+def random_tensors(cfg, seed, rank=8):
+    """bfloat16-representable float32 tensors: projections ~ N(0, 1.5 / sqrt(fan in)), norm weights around zero (plain ones around one),
+    decay inputs spread so that some channels forget within a few tokens and others keep hundreds"""
+    r = np.random.default_rng(seed)
+    out = {}
+    for name, shape in tensor_shapes(cfg, rank).items():
+        last = name.split(".")[-1]
+        if last in ("norm1", "norm1b", "norm2", "norm2b") or name in ("embed.norm", "final.norm"):
+            a = 0.2 * r.standard_normal(shape)
+        elif last == "norm":
+            a = 1.0 + 0.2 * r.standard_normal(shape)
+        elif name.endswith("a2.b"):
+            a = 2.0 + 2.0 * r.standard_normal(shape)
+        elif last == "dt_bias":
+            a = -2.0 + 1.5 * r.standard_normal(shape)
+        elif last == "A_log":
+            a = -1.0 + 0.7 * r.standard_normal(shape)
+        elif last == "b" and len(shape) == 1:
+            a = 0.3 * r.standard_normal(shape)
+        elif last == "conv":
+            a = 0.4 * r.standard_normal(shape) + 0.3
+        elif name in ("embed", "bigram"):
+            a = r.standard_normal(shape)
+        else:
+            a = 1.5 * r.standard_normal(shape) / math.sqrt(shape[-1])
+        out[name] = bf16_round(np.asarray(a, np.float32))
+    return out
