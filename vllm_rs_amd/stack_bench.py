@@ -1,5 +1,6 @@
-"""Throughput of a layer-stack model (Ditilix or Gaperax design) beside the dense bf16 Llama of the same widths —
-`python bench.py --design ditilix|gaperax`.
+"""Throughput of a layer-stack model (Ditilix, Gaperax or Zifetar design) beside the dense bf16 Llama of the same widths —
+`python bench.py --design ditilix|gaperax|zifetar` (Zifetar also beside the Ditilix mixture of experts of the same widths, the closest
+model of its class).
 
 Random weights of layer sizes that resemble a real model; for each size one JSON line with prefill tokens/s (one prompt of
 `prefill_tokens`, best of three engine steps) and decode tokens/s (batches of 1 and 8 behind 512-token prompts, HIP-event time of
@@ -75,6 +76,42 @@ def gaperax_costs(cj):
     return 2 * n, 2 * n
 
 
+def zifetar_config(width, heads, kv_heads, dim, layers, vocab, experts, top, expert_ff, chunk, rank):
+    """config.json dict of a Zifetar model: layers in the order parallel, delta rule, retention, ...; every layer a mixture of experts"""
+    rot = dict(base=5e5, dims=dim, scaling=dict(factor=8.0, low=1.0, high=4.0, original=8192))
+    par = dict(left=dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim, scale=dim ** -0.5, mask=dict(size=chunk), rot=rot),
+               right=dict(heads=heads // 2, dim=dim, vdim=dim, tau=16.0, rank_a=rank), left_scale=0.6, right_scale=0.9)
+    dl = dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim, conv=4, rank_a=rank, rank_g=rank)
+    ret = dict(heads=heads, dim=dim, vdim=dim, decay=[1.0 - 2.0 ** (-5.0 - 5.0 * h / max(heads - 1, 1)) for h in range(heads)], rot=dict(base=1e6, dims=dim))
+    mlp = dict(kind="moe", expert=dict(ff=expert_ff), router=dict(experts=experts, top=top))
+    kinds = [("parallel", par), ("channel_delta", dl), ("retention", ret)]
+    ls = [dict(type=kinds[i % 3][0], mixer=kinds[i % 3][1], mlp=mlp) for i in range(layers)]
+    return dict(architecture="Zifetar", width=width, vocab=vocab, norm=dict(eps=1e-6), embedding=dict(scale=width ** 0.5, bigram=dict(buckets=65521, mul_prev=31, mul_cur=7)),
+                layers=ls)
+
+
+def zifetar_costs(cj):
+    """(matrix FLOPs per token without attention and recurrences, weight bytes a one-token step reads) of a Zifetar config"""
+    W, n = cj["width"], 0
+    for layer in cj["layers"]:
+        mx = layer["mixer"]
+        if layer["type"] == "parallel":
+            le, ri = mx["left"], mx["right"]
+            H, G, D, V = le["heads"], le["kv_heads"], le["dim"], le["vdim"]
+            rh, rd, rv, ra = ri["heads"], ri["dim"], ri["vdim"], ri["rank_a"]
+            n += W * (H * D + G * D + G * V + rh * (2 * rd + 2 * rv) + ra) + ra * rh * rd + (H * V + rh * rv) * W
+        elif layer["type"] == "channel_delta":
+            H, G, D, V, ra, rg = mx["heads"], mx["kv_heads"], mx["dim"], mx["vdim"], mx["rank_a"], mx["rank_g"]
+            n += W * (2 * G * D + H * V + H + ra + rg) + ra * H * D + rg * H * V + H * V * W
+        else:
+            H, D, V = mx["heads"], mx["dim"], mx["vdim"]
+            n += W * (2 * H * D + 2 * H * V) + H * V * W
+        if layer.get("mlp"):
+            n += layer["mlp"]["router"]["top"] * 3 * W * layer["mlp"]["expert"]["ff"] + W * layer["mlp"]["router"]["experts"]
+    n += cj["vocab"] * W
+    return 2 * n, 2 * n
+
+
 def llama_costs(cfg):
     H, D = cfg["hidden_size"], cfg["head_dim"]
     per = H * (cfg["num_heads"] + 2 * cfg["num_kv_heads"]) * D + cfg["num_heads"] * D * H + 3 * H * cfg["intermediate_size"]
@@ -131,14 +168,25 @@ GAPERAX_SIZES = {
 }
 
 
+ZIFETAR_SIZES = {
+    # name: (width, heads, kv_heads, head size, layers, vocab, experts, top, expert ff, block mask, rank of the low-rank projections)
+    "zifetar-2048": (2048, 16, 4, 128, 3, 32000, 16, 2, 1024, 1024, 64),
+    "zifetar-4096": (4096, 32, 8, 128, 3, 32000, 16, 2, 2048, 1024, 128),
+}
+
+
 def main(steps=64, warmup=8, prefill_tokens=2048, graph=True, sizes=None, design="ditilix"):
     from . import _lib, checkpoint
     from .engine import BF16, Engine
     L = _lib.load()
     lines = []
-    table = GAPERAX_SIZES if design == "gaperax" else SIZES
+    table = GAPERAX_SIZES if design == "gaperax" else (ZIFETAR_SIZES if design == "zifetar" else SIZES)
     for name in (sizes or table):
-        if design == "gaperax":
+        if design == "zifetar":
+            width, heads, kvh, dim, layers, vocab, experts, top, eff, chunk, rank = table[name]
+            cj = zifetar_config(width, heads, kvh, dim, layers, vocab, experts, top, eff, chunk, rank)
+            ff = 4 * width
+        elif design == "gaperax":
             width, heads, kvh, dim, ff, layers, vocab, kr, qr, rd, window, keep_first = table[name]
             cj = gaperax_config(width, heads, kvh, dim, ff, layers, vocab, kr, qr, rd, window, keep_first)
         else:
@@ -147,7 +195,15 @@ def main(steps=64, warmup=8, prefill_tokens=2048, graph=True, sizes=None, design
         eng = Engine(checkpoint.parse_config(cj), num_gpu_blocks=512, max_num_seqs=8, max_model_len=4096, use_graph=graph).init_synthetic()
         res = dict(stack=measure(eng, L, vocab, prefill_tokens, steps, warmup))
         eng.close()
-        res["stack"]["flops_per_token"], res["stack"]["weight_bytes_per_step"] = gaperax_costs(cj) if design == "gaperax" else stack_costs(cj)
+        res["stack"]["flops_per_token"], res["stack"]["weight_bytes_per_step"] = (
+            zifetar_costs(cj) if design == "zifetar" else (gaperax_costs(cj) if design == "gaperax" else stack_costs(cj)))
+        if design == "zifetar":  # the closest model of the same class: softmax attention + the same mixture of experts in every layer
+            dj = stack_config(width, heads, kvh, dim, ff, layers + 1, vocab, experts, top, eff, 0, False)
+            dj["layers"] = dj["layers"][1:]
+            eng = Engine(checkpoint.parse_config(dj), num_gpu_blocks=512, max_num_seqs=8, max_model_len=4096, use_graph=graph).init_synthetic()
+            res["ditilix_moe"] = measure(eng, L, vocab, prefill_tokens, steps, warmup)
+            eng.close()
+            res["ditilix_moe"]["flops_per_token"], res["ditilix_moe"]["weight_bytes_per_step"] = stack_costs(dj)
         lcfg = dict(arch="llama", hidden_size=width, intermediate_size=ff, num_layers=layers, num_heads=heads, num_kv_heads=kvh, head_dim=dim,
                     vocab_size=vocab, max_position_embeddings=4096, rms_norm_eps=1e-5, rope_theta=10000.0, quant_method=None, dtype=BF16)
         eng = Engine(lcfg, num_gpu_blocks=512, max_num_seqs=8, max_model_len=4096, use_graph=graph).init_synthetic()
@@ -157,7 +213,7 @@ def main(steps=64, warmup=8, prefill_tokens=2048, graph=True, sizes=None, design
         for m in res.values():
             m["prefill_matrix_tflops"] = m["prefill_tokens_per_s"] * m["flops_per_token"] / 1e12
             m["decode_bs1_weight_gb_per_s"] = m["weight_bytes_per_step"] / (m["decode_bs1_ms_per_step"] / 1e3) / 1e9
-        line = dict(metric="stack_vs_dense_llama", size=name, design="Gaperax" if design == "gaperax" else "Ditilix", dtype="bf16", data="synthetic", prefill_tokens=prefill_tokens,
+        line = dict(metric="stack_vs_dense_llama", size=name, design={"gaperax": "Gaperax", "zifetar": "Zifetar"}.get(design, "Ditilix"), dtype="bf16", data="synthetic", prefill_tokens=prefill_tokens,
                     decode_context=512, steps=steps, **res)
         print(json.dumps(line), flush=True)
         lines.append(line)
