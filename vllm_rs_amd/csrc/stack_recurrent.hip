@@ -114,28 +114,37 @@ __global__ __launch_bounds__(256) void stk_sandwich_kernel(StkSandwichArgs a) {
   const T* rw = (const T*)a.router_w;
   for (int e = wave; e < a.n_router; e += 4) {
     float z = 0.f;
-    for (int c = lane; c < W; c += 64) z = fmaf(xs[c], El<T>::ld(rw + (size_t)e * W + c), z);
+    if (sizeof(T) == 2 && W % 8 == 0 && ((uintptr_t)rw % 16) == 0) {  // 8 weights a load; a lane's partial sums keep one order for a given W
+      for (int c = lane * 8; c < W; c += 64 * 8) {
+        const u32x4 v = *(const u32x4*)((const uint16_t*)rw + (size_t)e * W + c);
+        for (int i = 0; i < 4; i++) {
+          z = fmaf(xs[c + 2 * i], __uint_as_float(v[i] << 16), z);
+          z = fmaf(xs[c + 2 * i + 1], __uint_as_float(v[i] & 0xffff0000u), z);
+        }
+      }
+    } else {
+      for (int c = lane; c < W; c += 64) z = fmaf(xs[c], El<T>::ld(rw + (size_t)e * W + c), z);
+    }
     z = wave_sum(z);
     if (lane == 0) zs[e] = z + (a.router_bias ? a.router_bias[e] : 0.f);
   }
   __syncthreads();
-  if (tid == 0) {
-    float zmax = -INFINITY, sum = 0.f;
+  if (tid == 0) {  // the `top` largest in turn (ties: the lower index); a picked logit leaves the list
+    float zmax = 0.f, sum = 0.f;
     for (int j = 0; j < a.top; j++) {
-      int best = -1;
-      float bz = -INFINITY;
-      for (int e = 0; e < a.n_router; e++) {
-        bool taken = false;
-        for (int q = 0; q < j; q++) taken = taken || a.pair_expert[(size_t)t * a.top + q] == e;
-        if (!taken && (best < 0 || zs[e] > bz)) best = e, bz = zs[e];
-      }
-      a.pair_expert[(size_t)t * a.top + j] = best;
+      int best = 0;
+      float bz = zs[0];
+      for (int e = 1; e < a.n_router; e++)
+        if (zs[e] > bz) best = e, bz = zs[e];
+      zs[best] = -INFINITY;
       if (j == 0) zmax = bz;  // (the first pick is the largest logit)
       const float w = expf(bz - zmax);
+      a.pair_expert[(size_t)t * a.top + j] = best;
       a.pair_weight[(size_t)t * a.top + j] = w;
       sum += w;
     }
-    for (int j = 0; j < a.top; j++) a.pair_weight[(size_t)t * a.top + j] /= sum;
+    const float inv = 1.f / sum;
+    for (int j = 0; j < a.top; j++) a.pair_weight[(size_t)t * a.top + j] *= inv;
   }
 }
 
@@ -147,7 +156,7 @@ __global__ __launch_bounds__(256) void stk_head_prep_kernel(StkHeadPrepArgs a) {
   const float p = (float)a.positions[t];
   const int64_t slot = a.slots ? a.slots[t] : (int64_t)t;
   const int rp = a.rot.pairs;
-  for (int hh = wave; hh < a.Hq + a.Hk; hh += 4) {
+  for (int hh = blockIdx.y * 4 + wave; hh < a.Hq + a.Hk; hh += 4 * gridDim.y) {
     const bool is_q = hh < a.Hq;
     const int h = is_q ? hh : hh - a.Hq;
     if (!is_q && slot < 0) continue;
@@ -175,7 +184,7 @@ __global__ __launch_bounds__(256) void stk_head_prep_kernel(StkHeadPrepArgs a) {
   }
   if (a.v_out && slot >= 0) {
     TO* dst = (TO*)a.v_out + (size_t)slot * a.v_ld;
-    for (int c = threadIdx.x; c < a.nv; c += 256) El<TO>::st(dst + c, raw[a.v_off + c]);
+    for (int c = blockIdx.y * 256 + threadIdx.x; c < a.nv; c += 256 * gridDim.y) El<TO>::st(dst + c, raw[a.v_off + c]);
   }
 }
 
@@ -192,16 +201,25 @@ __global__ __launch_bounds__(256) void stk_delta_prep_kernel(StkDeltaPrepArgs a)
   const int i = t - t0;                                   // place of the row in its sequence's part of the step
   const bool fresh = a.positions[t0] == 0;                // the sequence starts in this step: nothing before its first row
   const float* cs = a.conv_state + (size_t)slot * (taps - 1) * C;
-  for (int c = tid; c < C; c += 256) {
-    float y = 0.f;
+  // tap j of a row reads the input taps - 1 - j places back: a row of this step, the slot's kept inputs, or nothing (a sequence's start).
+  // Every address is valid whatever the case (the weight of a load that does not count is 0), so no load waits for a branch; four
+  // channels go side by side.
+  for (int c0 = tid; c0 < C; c0 += 4 * 256) {
+    float y[4] = {0.f, 0.f, 0.f, 0.f};
     for (int j = 0; j < taps; j++) {
       const int e = i - (taps - 1) + j;
-      float in = 0.f;
-      if (e >= 0) in = a.raw[(size_t)(t0 + e) * a.ld + c];
-      else if (!fresh) in = cs[(size_t)(taps - 1 + e) * C + c];
-      y = fmaf(a.conv_w[(size_t)c * taps + j], in, y);
+      const bool from_step = e >= 0, counts = from_step || (!fresh && taps > 1);
+      const float* src = from_step ? a.raw + (size_t)(t0 + e) * a.ld : (counts ? cs + (size_t)(taps - 1 + e) * C : a.raw + (size_t)t * a.ld);
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        const int c = min(c0 + u * 256, C - 1);
+        const float wv = counts ? a.conv_w[(size_t)c * taps + j] : 0.f;
+        y[u] = fmaf(wv, src[c], y[u]);
+      }
     }
-    ys[c] = siluf_(y);
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+      if (c0 + u * 256 < C) ys[c0 + u * 256] = siluf_(y[u]);
   }
   __syncthreads();
   float* out = a.qkv_out + (size_t)t * C;
@@ -250,11 +268,31 @@ __global__ __launch_bounds__(256) void stk_sigmoid_pow_kernel(const float* z, in
 // neighbouring lanes, R rows each, in registers for the whole step.  Sums over the rows (S^T k, S^T q) add a lane's R products in order,
 // then the P lanes by xor shuffles: an order fixed by `dim` alone.  q, k and the decays of TT tokens are staged in LDS once for all
 // columns.
-template <int R>
-__global__ __launch_bounds__(256) void stk_linear_scan_kernel(StkScanArgs a, int P) {
-  constexpr int TT = 16;
-  extern __shared__ float lds[];
-  const int dim = a.dim, vdim = a.vdim, dimP = P * R, CPB = 256 / P;
+// sum over the P neighbouring lanes that share a column (P a power of two, lanes aligned to P), left in all of them.  Inside a row of 16
+// lanes the partner comes by DPP (quad permutes, then mirrors of half a row and of a row: after each step the lanes of a group hold one
+// value, so a mirror is as good as an xor); beyond 16 lanes by a cross-lane read.  One fixed order for a given P.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+template <int P>
+__device__ __forceinline__ float group_sum(float v) {
+  if (P >= 2) v += dpp_f32<0xB1>(v);    // quad_perm [1, 0, 3, 2]
+  if (P >= 4) v += dpp_f32<0x4E>(v);    // quad_perm [2, 3, 0, 1]
+  if (P >= 8) v += dpp_f32<0x141>(v);   // row_half_mirror
+  if (P >= 16) v += dpp_f32<0x140>(v);  // row_mirror
+  if (P >= 32) v += __shfl_xor(v, 16, 64);
+  return v;
+}
+
+// P, the presence of per-row decays and of the delta rule are template parameters: the 16 tokens of a tile are one straight line of code, so
+// the LDS reads of the tokens ahead are in flight while a token's sums run.
+template <int R, int P, bool DECAY, bool BETA>
+__global__ __launch_bounds__(256) void stk_linear_scan_kernel(StkScanArgs a) {
+  constexpr int TT = 16, NL = 4;     // tokens a tile; 16-byte loads a thread and array for one tile (TT * dimP / 4 / 256, dimP <= 256)
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  constexpr int dimP = P * R, CPB = 256 / P, d4n = dimP / 4;
+  const int dim = a.dim, vdim = a.vdim;
   float* ks = lds;                   // [TT][dimP]
   float* qs = ks + TT * dimP;        // [TT][dimP]
   float* ds = qs + TT * dimP;        // [TT][dimP]
@@ -272,51 +310,117 @@ __global__ __launch_bounds__(256) void stk_linear_scan_kernel(StkScanArgs a, int
 #pragma unroll
   for (int j = 0; j < R; j++) S[j] = (!fresh && col && r * R + j < dim) ? sp[j] : 0.f;
   const float hd = a.head_decay ? a.head_decay[h] : 1.f;
+  // rows of dim floats that start on 16 bytes are fetched four floats a load
+  const bool vec = dim % 4 == 0 && a.ldk % 4 == 0 && a.ldq % 4 == 0 && (!DECAY || a.ldd % 4 == 0) && ((uintptr_t)a.k % 16) == 0 && ((uintptr_t)a.q % 16) == 0 &&
+                   (!DECAY || ((uintptr_t)a.decay % 16) == 0);
+  // A tile's q, k, decays, values and write strengths travel global memory -> registers -> LDS; the registers of the NEXT tile are requested
+  // before the current tile's tokens run, so their way from memory lies beside the arithmetic.
+  float4 kn[NL], qn[NL], dn[NL];
+  float vbuf[16], bn = 0.f;
+  constexpr int vcount = TT * CPB;     // values of a tile: a thread takes elements tid, tid + 256, ... (at most 16)
+  auto row4 = [&](const float* base, int ld, int hh, size_t t, int d, float fill) {
+    const float* p = base + t * ld + hh * dim + d;
+    if (vec && d + 3 < dim) return *(const float4*)p;
+    float4 o;
+    o.x = d < dim ? p[0] : fill, o.y = d + 1 < dim ? p[1] : fill, o.z = d + 2 < dim ? p[2] : fill, o.w = d + 3 < dim ? p[3] : fill;
+    return o;
+  };
+  auto request = [&](int i0) {
+    const int nt = min(TT, n - i0);
+#pragma unroll
+    for (int u = 0; u < NL; u++) {
+      const int e = tid + u * 256, i = e / d4n, d = (e % d4n) * 4;
+      kn[u] = qn[u] = make_float4(0.f, 0.f, 0.f, 0.f), dn[u] = make_float4(1.f, 1.f, 1.f, 1.f);
+      if (e < TT * d4n && i < nt) {
+        const size_t t = (size_t)(t0 + i0 + i);
+        kn[u] = row4(a.k, a.ldk, hq, t, d, 0.f);
+        qn[u] = row4(a.q, a.ldq, hq, t, d, 0.f);
+        if (DECAY) dn[u] = row4(a.decay, a.ldd, h, t, d, 1.f);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 16; u++) {
+      const int e = tid + u * 256;
+      if (e < vcount) {
+        const int i = e / CPB, cc = blockIdx.x * CPB + e % CPB;
+        vbuf[u] = (i < nt && cc < vdim) ? a.v[(size_t)(t0 + i0 + i) * a.ldv + h * vdim + cc] : 0.f;
+      }
+    }
+    if (BETA && tid < nt) bn = a.beta[(size_t)(t0 + i0 + tid) * a.ldb + h];
+  };
+  auto deposit = [&]() {
+#pragma unroll
+    for (int u = 0; u < NL; u++) {
+      const int e = tid + u * 256;
+      if (e < TT * d4n) {
+        *(float4*)(ks + e * 4) = kn[u];
+        float4 qv = qn[u];
+        qv.x *= a.q_scale, qv.y *= a.q_scale, qv.z *= a.q_scale, qv.w *= a.q_scale;
+        *(float4*)(qs + e * 4) = qv;
+        if (DECAY) *(float4*)(ds + e * 4) = dn[u];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 16; u++) {
+      const int e = tid + u * 256;
+      if (e < vcount) vs[e] = vbuf[u];
+    }
+    if (BETA && tid < TT) bs[tid] = bn;
+  };
+  request(0);
   for (int i0 = 0; i0 < n; i0 += TT) {
     const int nt = min(TT, n - i0);
     __syncthreads();
-    for (int e = tid; e < nt * dimP; e += 256) {
-      const int i = e / dimP, d = e % dimP;
-      const size_t t = (size_t)(t0 + i0 + i);
-      const bool in = d < dim;
-      ks[e] = in ? a.k[t * a.ldk + hq * dim + d] : 0.f;
-      qs[e] = in ? a.q[t * a.ldq + hq * dim + d] * a.q_scale : 0.f;
-      if (a.decay) ds[e] = in ? a.decay[t * a.ldd + h * dim + d] : 1.f;
-    }
-    for (int e = tid; e < nt * CPB; e += 256) {
-      const int i = e / CPB, cc = blockIdx.x * CPB + e % CPB;
-      vs[e] = cc < vdim ? a.v[(size_t)(t0 + i0 + i) * a.ldv + h * vdim + cc] : 0.f;
-    }
-    if (a.beta)
-      for (int i = tid; i < nt; i += 256) bs[i] = a.beta[(size_t)(t0 + i0 + i) * a.ldb + h];
+    deposit();
     __syncthreads();
-    for (int i = 0; i < nt; i++) {
-      const float* kr = ks + i * dimP + r * R;
-      const float* qr = qs + i * dimP + r * R;
-      if (a.decay) {
-        const float* dr = ds + i * dimP + r * R;
+    if (i0 + TT < n) request(i0 + TT);
+    // a token's operands come from LDS one token ahead of its arithmetic (two register sets, 16-byte reads)
+    float kv[2][R], qv[2][R], dv[2][R], uv[2], bv[2];
+    auto fetch = [&](int i, int w) {
 #pragma unroll
-        for (int j = 0; j < R; j++) S[j] *= dr[j];
-      } else {
-#pragma unroll
-        for (int j = 0; j < R; j++) S[j] *= hd;
+      for (int j = 0; j < R; j += 4) {
+        const float4 k4 = *(const float4*)(ks + i * dimP + r * R + j), q4 = *(const float4*)(qs + i * dimP + r * R + j);
+        kv[w][j] = k4.x, kv[w][j + 1] = k4.y, kv[w][j + 2] = k4.z, kv[w][j + 3] = k4.w;
+        qv[w][j] = q4.x, qv[w][j + 1] = q4.y, qv[w][j + 2] = q4.z, qv[w][j + 3] = q4.w;
+        if (DECAY) {
+          const float4 d4 = *(const float4*)(ds + i * dimP + r * R + j);
+          dv[w][j] = d4.x, dv[w][j + 1] = d4.y, dv[w][j + 2] = d4.z, dv[w][j + 3] = d4.w;
+        }
       }
-      float u = vs[i * CPB + cl];
-      if (a.beta) {
-        float dot = 0.f;
+      uv[w] = vs[i * CPB + cl];
+      if (BETA) bv[w] = bs[i];
+    };
+    auto token = [&](int i, int w) {
 #pragma unroll
-        for (int j = 0; j < R; j++) dot = fmaf(S[j], kr[j], dot);
-        for (int o = 1; o < P; o <<= 1) dot += __shfl_xor(dot, o, 64);
-        u = bs[i] * (u - dot);
-      }
-      float o_ = 0.f;
+      for (int j = 0; j < R; j++) S[j] *= DECAY ? dv[w][j] : hd;
+      float u = uv[w];
+      if (BETA) {
+        float d0 = 0.f, d1 = 0.f;  // (two chains; their sum order is fixed)
 #pragma unroll
-      for (int j = 0; j < R; j++) {
-        S[j] = fmaf(kr[j], u, S[j]);
-        o_ = fmaf(S[j], qr[j], o_);
+        for (int j = 0; j < R; j += 2) d0 = fmaf(S[j], kv[w][j], d0), d1 = fmaf(S[j + 1], kv[w][j + 1], d1);
+        u = bv[w] * (u - group_sum<P>(d0 + d1));
       }
-      for (int o = 1; o < P; o <<= 1) o_ += __shfl_xor(o_, o, 64);
+      float o0 = 0.f, o1 = 0.f;
+#pragma unroll
+      for (int j = 0; j < R; j += 2) {
+        S[j] = fmaf(kv[w][j], u, S[j]), S[j + 1] = fmaf(kv[w][j + 1], u, S[j + 1]);
+        o0 = fmaf(S[j], qv[w][j], o0), o1 = fmaf(S[j + 1], qv[w][j + 1], o1);
+      }
+      const float o_ = group_sum<P>(o0 + o1);
       if (r == 0 && col) a.out[(size_t)(t0 + i0 + i) * a.ldo + h * vdim + c] = o_;
+    };
+    fetch(0, 0);
+    if (nt == TT) {
+#pragma unroll
+      for (int i = 0; i < TT; i++) {
+        if (i + 1 < TT) fetch(i + 1, (i + 1) & 1);
+        token(i, i & 1);
+      }
+    } else {
+      for (int i = 0; i < nt; i++) {
+        fetch(i, 0);
+        token(i, 0);
+      }
     }
   }
   if (col)
@@ -372,8 +476,9 @@ void vra_stack_head_prep(const StkHeadPrepArgs& a, int dtype, int64_t stream) {
   VRA_CHECK_ARG(a.raw && a.positions && a.T > 0 && a.dim > 0 && a.Hq >= 0 && a.Hk >= 0 && (a.Hq == 0 || a.q_out) && (a.Hk == 0 || a.k_out),
                 "stack head prep: null pointer or empty shape");
   VRA_CHECK_ARG(2 * a.rot.pairs <= a.dim && (a.rot.pairs == 0 || a.rot.freq_hi), "stack head prep: more rotated dimensions than the head has");
-  if (a.out_f32 || dtype == VRA_F32) launch_checked("stack head prep", [&] { stk_head_prep_kernel<float><<<a.T, 256, 0, as_stream(stream)>>>(a); });
-  else launch_checked("stack head prep", [&] { stk_head_prep_kernel<uint16_t><<<a.T, 256, 0, as_stream(stream)>>>(a); });
+  const dim3 grid(a.T, std::min((a.Hq + a.Hk + 3) / 4, 64));  // a head per wave
+  if (a.out_f32 || dtype == VRA_F32) launch_checked("stack head prep", [&] { stk_head_prep_kernel<float><<<grid, 256, 0, as_stream(stream)>>>(a); });
+  else launch_checked("stack head prep", [&] { stk_head_prep_kernel<uint16_t><<<grid, 256, 0, as_stream(stream)>>>(a); });
 }
 
 void vra_stack_delta_prep(const StkDeltaPrepArgs& a, int64_t stream) {
@@ -407,7 +512,24 @@ void vra_stack_linear_scan(const StkScanArgs& a, int64_t stream) {
   const int CPB = 256 / P, dimP = P * R;
   const size_t lds = ((size_t)16 * dimP * 3 + (size_t)16 * CPB + 16) * sizeof(float);
   dim3 grid((a.vdim + CPB - 1) / CPB, a.H, a.B);
-  launch_checked("stack linear scan", [&] { stk_linear_scan_kernel<R><<<grid, 256, lds, as_stream(stream)>>>(a, P); });
+  hipStream_t st = as_stream(stream);
+  const bool decay = a.decay != nullptr, beta = a.beta != nullptr;
+  VRA_CHECK_ARG(decay || !beta, "stack linear scan: the delta rule comes with per-row decays");
+#define STK_SCAN(PV)                                                                                                            \
+  launch_checked("stack linear scan", [&] {                                                                                     \
+    if (beta) stk_linear_scan_kernel<R, PV, true, true><<<grid, 256, lds, st>>>(a);                                             \
+    else if (decay) stk_linear_scan_kernel<R, PV, true, false><<<grid, 256, lds, st>>>(a);                                      \
+    else stk_linear_scan_kernel<R, PV, false, false><<<grid, 256, lds, st>>>(a);                                                \
+  })
+  switch (P) {
+    case 1: STK_SCAN(1); break;
+    case 2: STK_SCAN(2); break;
+    case 4: STK_SCAN(4); break;
+    case 8: STK_SCAN(8); break;
+    case 16: STK_SCAN(16); break;
+    default: STK_SCAN(32); break;
+  }
+#undef STK_SCAN
 }
 
 void vra_stack_head_norm_gate(const float* o, const float* w, const float* gate, int gate_ld, int gate_act, float eps, void* out, int T, int H, int vdim,
