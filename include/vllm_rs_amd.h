@@ -683,6 +683,24 @@ void vra_stack_op_attention_ex(const void* q, int32_t ldq, void* out, const void
                                int32_t max_q, int32_t H, int32_t G, int32_t dim, int32_t vdim, int32_t BS, int32_t max_blocks,
                                float scale, const float* sink, int32_t k_ld, int32_t v_ld, int32_t dtype, int64_t stream);
 
+/* Operators of sandwich-norm stacks with recurrent mixers (csrc/stack_recurrent.hip; csrc/stack_launch.h says what each computes).
+ * attention_chunk: vra_stack_op_attention_ex with visibility restricted to the query's own block of `chunk` positions.
+ * linear_scan: S <- diag(d_t) S; u = v_t or beta_t (v_t - S^T k_t); S <- S + k_t u^T; o_t = S^T (q_scale q_t), the state of sequence b in
+ * slot state_slots[b] ([slots, H, vdim, dim] f32), zeros for a sequence whose first row stands at position 0.
+ * sandwich_norm: x += N(c1 sum_j pw_j p1_j + c2 p2; post_w); h = N(x; pre_w); router = biased logits on h, top-k, softmax over the chosen. */
+void vra_stack_op_attention_chunk(const void* q, int32_t ldq, void* out, const void* kc, const void* vc, const int64_t* positions,
+                                  const uint32_t* block_tables, const uint32_t* context_lens, const uint32_t* cu_q, int32_t B, int32_t T,
+                                  int32_t max_q, int32_t H, int32_t G, int32_t dim, int32_t vdim, int32_t BS, int32_t max_blocks,
+                                  float scale, int32_t chunk, int32_t dtype, int64_t stream);
+void vra_stack_op_linear_scan(const float* q, int32_t ldq, const float* k, int32_t ldk, const float* v, int32_t ldv, const float* decay,
+                              int32_t ldd, const float* head_decay, const float* beta, int32_t ldb, float q_scale, float* state,
+                              const int32_t* state_slots, const int64_t* positions, const uint32_t* cu_q, float* out, int32_t ldo,
+                              int32_t B, int32_t H, int32_t qk_rep, int32_t dim, int32_t vdim, int64_t stream);
+void vra_stack_op_sandwich_norm(float* x, const float* p1, int32_t n1, const float* pw, float c1, const float* p2, float c2,
+                                const float* post_w, const float* pre_w, void* h, float eps, int32_t T, int32_t W, const void* router_w,
+                                const float* router_bias, int32_t n_router, int32_t top, int32_t* pair_expert, float* pair_weight,
+                                int32_t dtype, int64_t stream);
+
 /* decode-step microbenchmark hook used by bench.py: runs `steps` decode steps of the current
  * running batch back to back (graph replay when enabled) and returns elapsed ms measured with HIP
  * events on the engine stream; tokens are sampled and appended exactly as in vra_engine_step. */

@@ -5,6 +5,7 @@ f32 models must agree with the oracle to f32 rounding, bf16 models to bf16 round
 its prompt was cut, on the rest of the batch or on the pages and state slots it got.
 """
 import json
+import math
 import os
 import struct
 import subprocess
@@ -445,3 +446,182 @@ def test_trace_runner_on_a_model_folder(tmp_path):
         got = [np.fromfile(out / ("%d.f32" % i), "<f4").reshape(-1, cfg["vocab"]) for i in range(5)]
         assert [g.shape[0] for g in got] == [w.shape[0] for w in want]
         agree(np.concatenate(got), np.concatenate(want), dt, dtype)
+
+
+# ------------------------------------------------------------------------------------------------ operators alone, planted values
+from tests.test_gpu_stack import check, empty, from_dev, paged, raw, to_dev  # noqa: E402
+from vllm_rs_amd import _lib  # noqa: E402
+
+
+def masked_softmax(q, k, v, scale, vis):
+    """q [Tq, H, D] against ALL keys k [Tk, G, D] under the visibility matrix vis [Tq, Tk] (the oracle's attention takes square prompts)"""
+    Tq, H, _ = q.shape
+    G = k.shape[1]
+    out = np.zeros((Tq, H, v.shape[-1]))
+    for hd in range(H):
+        g = hd // (H // G)
+        s = np.where(vis, (q[:, hd] @ k[:, g].T) * scale, -np.inf)
+        e = np.exp(s - s.max(-1, keepdims=True))
+        out[:, hd] = (e / e.sum(-1, keepdims=True)) @ v[:, g]
+    return out
+
+
+def run_masked_attention(L, q, positions, k, v, scale, chunk, dt, decode, r, BS=64):
+    Tq, H, dim = q.shape
+    G, vdim = k.shape[1], v.shape[2]
+    kc, vc, table = paged(k, v, BS, r, dt)
+    if decode:
+        res = []
+        for i in range(Tq):
+            o1 = empty(H * vdim * 4)
+            qi = to_dev(q[i].reshape(1, H * dim), dt)
+            L.vra_stack_op_attention_chunk(qi.ptr, H * dim, o1.ptr, kc.ptr, vc.ptr, raw([positions[i]], np.int64).ptr, raw(table, np.uint32).ptr,
+                                           raw([positions[i] + 1], np.uint32).ptr, None, 1, 1, 1, H, G, dim, vdim, BS, len(table), scale, chunk, dt, 0)
+            check()
+            res.append(from_dev(o1, (H, vdim), dt))
+        return np.stack(res)
+    out = empty(Tq * H * vdim * 4)
+    L.vra_stack_op_attention_chunk(to_dev(q.reshape(Tq, H * dim), dt).ptr, H * dim, out.ptr, kc.ptr, vc.ptr, raw(positions, np.int64).ptr,
+                                   raw(table, np.uint32).ptr, raw([k.shape[0]], np.uint32).ptr, raw([0, Tq], np.uint32).ptr, 1, Tq, Tq, H, G, dim, vdim, BS,
+                                   len(table), scale, chunk, dt, 0)
+    check()
+    return from_dev(out, (Tq, H, vdim), dt)
+
+
+@pytest.mark.parametrize("dt", [F32, BF16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("decode", [False, True], ids=["prompt", "decoded"])
+@pytest.mark.parametrize("chunk,dim,vdim", [(200, 32, 16), (64, 16, 8), (70, 64, 64), (1, 16, 8)])
+def test_block_mask_planted_key(dt, decode, chunk, dim, vdim):
+    """one key stands out among 900 (its value is a marker).  A query in the key's own block of positions and not before it returns the
+    marker — at the block's first and last position, across page borders; a query of the next block, or of the block before, or before
+    the key inside its block, does not feel it at all.  (bf16 prompts: matrix-core kernel for the first and third shape, FMA otherwise.)"""
+    L = _lib.load()
+    r = np.random.default_rng(chunk + dim)
+    Tk, H, G = 900, 4, 2
+    base_k = zo.bf16_round((0.1 * r.standard_normal((Tk, G, dim))).astype(np.float32))
+    base_v = zo.bf16_round((0.1 * r.standard_normal((Tk, G, vdim))).astype(np.float32))
+    u = np.zeros(dim, np.float32)
+    u[3] = 1.0
+    for j in (0, chunk - 1, chunk, 3 * chunk + chunk // 2, (899 // chunk) * chunk):
+        if j >= Tk:
+            continue
+        k, v = base_k.copy(), base_v.copy()
+        k[j, :, :] = 16.0 * u  # score 8 * 16 * 0.25 = 32 against |scores| < 1 elsewhere
+        v[j, :, :] = 5.0
+        lo, hi = j // chunk * chunk, min((j // chunk + 1) * chunk, Tk)
+        positions = sorted({p for p in (lo - 1, lo, j - 1, j, j + 1, hi - 1, hi, hi + 1, 899) if 0 <= p < Tk})
+        q = np.tile(8.0 * u, (len(positions), H, 1)).astype(np.float32)
+        got = run_masked_attention(L, q, np.array(positions, np.int64), k, v, 0.25, chunk, dt, decode, r)
+        for i, p in enumerate(positions):
+            sees = lo <= j <= p < hi
+            if sees:
+                assert np.abs(got[i] - 5.0).max() < 2e-2, (j, p)
+            else:
+                assert np.abs(got[i]).max() < 1.0, (j, p)  # (small values only: the marker has no weight at all)
+        vis = np.array([[(kk <= p) and (kk // chunk == p // chunk) for kk in range(Tk)] for p in positions])
+        ref = masked_softmax(q.astype(np.float64), k.astype(np.float64), v.astype(np.float64), 0.25, vis)
+        assert rel(got, ref) < (2e-5 if dt == F32 else 6e-3)
+
+
+def run_scan(L, q, k, v, decay, head_decay, beta, q_scale, cuts, slots, state, n_slots, qk_rep=1):
+    """the recurrence over ONE sequence given in portions `cuts`, its state in slot `slots` of `state` (a device buffer that persists)"""
+    T, Hq, D = q.shape
+    H, V = v.shape[1], v.shape[2]
+    outs, at = [], 0
+    for c in cuts:
+        sl = slice(at, at + c)
+        out = empty(c * H * V * 4)
+        f = lambda a: raw(np.ascontiguousarray(a[sl].reshape(c, -1)), np.float32).ptr
+        L.vra_stack_op_linear_scan(f(q), Hq * D, f(k), Hq * D, f(v), H * V, f(decay) if decay is not None else None, H * D,
+                                   raw(head_decay, np.float32).ptr if head_decay is not None else None, f(beta) if beta is not None else None, H, q_scale,
+                                   state.ptr, raw([slots], np.int32).ptr, raw(np.arange(at, at + c), np.int64).ptr, raw([0, c], np.uint32).ptr if c > 1 or at == 0 else None,
+                                   out.ptr, H * V, 1, H, qk_rep, D, V, 0)
+        check()
+        outs.append(out.numpy(np.float32, (c, H, V)))
+        at += c
+    return np.concatenate(outs)
+
+
+@pytest.mark.parametrize("form", ["head-decay", "row-decay", "delta"])
+@pytest.mark.parametrize("H,rep,D,V", [(2, 1, 8, 8), (3, 1, 5, 7), (4, 2, 16, 24), (2, 1, 64, 40), (2, 2, 128, 128), (1, 1, 200, 9), (2, 1, 24, 300)])
+def test_linear_recurrence_alone(form, H, rep, D, V):
+    """the recurrence kernel against the oracle's token loop: every lane grouping (key sizes 5 .. 200), value sizes off the workgroup's
+    column count, grouped q / k heads; one whole step, and portions (down to one token, with single-token steps in the decode form) whose
+    state waits in a slot that held another sequence's state before"""
+    L = _lib.load()
+    r = np.random.default_rng(D * 7 + V)
+    T = 75
+    q = r.standard_normal((T, H // rep, D)).astype(np.float32)
+    k = (r.standard_normal((T, H // rep, D)) / math.sqrt(D)).astype(np.float32)
+    v = r.standard_normal((T, H, V)).astype(np.float32)
+    decay = head_decay = beta = None
+    if form == "head-decay":
+        head_decay = (0.8 + 0.19 * r.random(H)).astype(np.float32)
+        dd = np.broadcast_to(head_decay[None, :, None], (T, H, D))
+    else:
+        decay = (0.7 + 0.3 * r.random((T, H, D))).astype(np.float32)
+        dd = decay
+    if form == "delta":
+        beta = r.random((T, H)).astype(np.float32)
+        k = k / np.sqrt((k * k).sum(-1, keepdims=True))
+    ref = zo.linear_recurrence(np.repeat(q, rep, 1).astype(np.float64) * 0.5, np.repeat(k, rep, 1).astype(np.float64), v.astype(np.float64),
+                               np.asarray(dd, np.float64), None if beta is None else beta.astype(np.float64))
+    n_slots = 3
+    state = raw(r.standard_normal(n_slots * H * V * D).astype(np.float32) * 100.0, np.float32)  # (what earlier sequences left: must not be felt)
+    whole = run_scan(L, q, k, v, decay, head_decay, beta, 0.5, [T], 1, state, n_slots, rep)
+    assert rel(whole, ref) < 1e-5
+    parts = run_scan(L, q, k, v, decay, head_decay, beta, 0.5, [1, 1, 2, 16, 1, 17, 32, 1, 4], 2, state, n_slots, rep)
+    assert rel(parts, ref) < 1e-5 and np.abs(parts - whole).max() <= 1e-6 * np.abs(whole).max()
+    again = run_scan(L, q, k, v, decay, head_decay, beta, 0.5, [40, 35], 1, state, n_slots, rep)  # the slot of the first run, used again
+    assert rel(again, ref) < 1e-5
+
+
+
+@pytest.mark.parametrize("dt", [F32, BF16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("W,E,top", [(96, 5, 2), (51, 3, 3), (256, 40, 1), (64, 8, 4)])
+def test_seam_norms_and_router(dt, W, E, top):
+    """x += N(c1 sum_j w_j part_j + c2 part2; post), h = N(x; pre), router: biased logits on h, the `top` largest, softmax over those alone.
+    One logit is planted far above the rest in some rows (its weight is then 1 up to e^-20) and two equal logits in another (the lower index wins)."""
+    L = _lib.load()
+    r = np.random.default_rng(W + E)
+    T, n1, eps = 9, 3, 1e-5
+    x = r.standard_normal((T, W)).astype(np.float32)
+    p1 = r.standard_normal((T * n1, W)).astype(np.float32)
+    pw = r.random(T * n1).astype(np.float32)
+    p2 = r.standard_normal((T, W)).astype(np.float32)
+    post, pre = (1 + 0.2 * r.standard_normal(W)).astype(np.float32), (1 + 0.2 * r.standard_normal(W)).astype(np.float32)
+    rw = zo.bf16_round((r.standard_normal((E, W)) / math.sqrt(W)).astype(np.float32))
+    rb = (0.3 * r.standard_normal(E)).astype(np.float32)
+    s = 0.6 * (pw[:, None] * p1).reshape(T, n1, W).sum(1).astype(np.float64) + 0.9 * p2
+    x_ref = x + zo.rms(s, eps) * post
+    h_ref = zo.rms(x_ref, eps) * pre
+    z = h_ref @ rw.T.astype(np.float64) + rb
+    xd, hd = raw(x, np.float32), empty(T * W * 4)
+    pe, pwt = empty(T * top * 4), empty(T * top * 4)
+    L.vra_stack_op_sandwich_norm(xd.ptr, raw(p1, np.float32).ptr, n1, raw(pw, np.float32).ptr, 0.6, raw(p2, np.float32).ptr, 0.9, raw(post, np.float32).ptr,
+                                 raw(pre, np.float32).ptr, hd.ptr, eps, T, W, to_dev(rw, dt).ptr, raw(rb, np.float32).ptr, E, top, pe.ptr, pwt.ptr, dt, 0)
+    check()
+    assert rel(xd.numpy(np.float32, (T, W)), x_ref) < 1e-6
+    assert rel(from_dev(hd, (T, W), dt), h_ref) < (1e-6 if dt == F32 else 4e-3)
+    experts, weights = pe.numpy(np.int32, (T, top)), pwt.numpy(np.float32, (T, top))
+    for t in range(T):
+        order = np.argsort(-z[t], kind="stable")[:top]
+        gap = np.sort(z[t])[::-1]
+        if top < E and gap[top - 1] - gap[top] < 1e-3:
+            continue  # (a close call at the cut: either choice is right to rounding)
+        assert sorted(experts[t].tolist()) == sorted(order.tolist()), t
+        e = np.exp(z[t, experts[t]] - z[t, experts[t]].max())
+        assert np.allclose(weights[t], e / e.sum(), atol=2e-5 if dt == F32 else 2e-2) and abs(weights[t].sum() - 1.0) < 1e-5
+    # a towering logit takes all the weight; equal logits go to the lower index
+    big = rb.copy()
+    big[E - 1] = 40.0
+    L.vra_stack_op_sandwich_norm(xd.ptr, None, 1, None, 1.0, None, 1.0, None, raw(pre, np.float32).ptr, hd.ptr, eps, T, W, to_dev(np.zeros((E, W), np.float32), dt).ptr,
+                                 raw(big, np.float32).ptr, E, top, pe.ptr, pwt.ptr, dt, 0)
+    check()
+    experts, weights = pe.numpy(np.int32, (T, top)), pwt.numpy(np.float32, (T, top))
+    assert (experts[:, 0] == E - 1).all() and (weights[:, 0] > 1.0 - 1e-6 * top).all()
+    L.vra_stack_op_sandwich_norm(xd.ptr, None, 1, None, 1.0, None, 1.0, None, raw(pre, np.float32).ptr, hd.ptr, eps, T, W, to_dev(np.zeros((E, W), np.float32), dt).ptr,
+                                 raw(np.zeros(E, np.float32), np.float32).ptr, E, top, pe.ptr, pwt.ptr, dt, 0)
+    check()
+    experts, weights = pe.numpy(np.int32, (T, top)), pwt.numpy(np.float32, (T, top))
+    assert (experts == np.arange(top)[None, :]).all() and np.allclose(weights, 1.0 / top)

@@ -542,3 +542,33 @@ void vra_stack_head_norm_gate(const float* o, const float* w, const float* gate,
       stk_head_norm_gate_kernel<uint16_t><<<T, 256, 0, as_stream(stream)>>>(o, w, gate, gate_ld, gate_act, eps, (uint16_t*)out, H, vdim);
     });
 }
+
+// ================================================================================================ C entry points (operator tests)
+extern "C" void vra_stack_op_attention_chunk(const void* q, int32_t ldq, void* out, const void* kc, const void* vc, const int64_t* positions,
+                                             const uint32_t* block_tables, const uint32_t* context_lens, const uint32_t* cu_q, int32_t B, int32_t T,
+                                             int32_t max_q, int32_t H, int32_t G, int32_t dim, int32_t vdim, int32_t BS, int32_t max_blocks, float scale,
+                                             int32_t chunk, int32_t dtype, int64_t stream) {
+  StkAttnArgs a;
+  a.q = q, a.ldq = ldq, a.out = out, a.kc = kc, a.vc = vc, a.positions = positions, a.block_tables = block_tables, a.context_lens = context_lens;
+  a.cu_q = cu_q, a.B = B, a.T = T, a.max_q = max_q, a.H = H, a.G = G, a.dim = dim, a.vdim = vdim, a.BS = BS, a.max_blocks = max_blocks;
+  a.scale = scale, a.chunk = chunk;
+  vra_stack_attention(a, dtype, stream);
+}
+extern "C" void vra_stack_op_linear_scan(const float* q, int32_t ldq, const float* k, int32_t ldk, const float* v, int32_t ldv, const float* decay, int32_t ldd,
+                                         const float* head_decay, const float* beta, int32_t ldb, float q_scale, float* state, const int32_t* state_slots,
+                                         const int64_t* positions, const uint32_t* cu_q, float* out, int32_t ldo, int32_t B, int32_t H, int32_t qk_rep,
+                                         int32_t dim, int32_t vdim, int64_t stream) {
+  StkScanArgs a;
+  a.q = q, a.ldq = ldq, a.k = k, a.ldk = ldk, a.v = v, a.ldv = ldv, a.decay = decay, a.ldd = ldd, a.head_decay = head_decay, a.beta = beta, a.ldb = ldb;
+  a.q_scale = q_scale, a.state = state, a.state_slots = state_slots, a.positions = positions, a.cu_q = cu_q, a.out = out, a.ldo = ldo;
+  a.B = B, a.H = H, a.qk_rep = qk_rep, a.dim = dim, a.vdim = vdim;
+  vra_stack_linear_scan(a, stream);
+}
+extern "C" void vra_stack_op_sandwich_norm(float* x, const float* p1, int32_t n1, const float* pw, float c1, const float* p2, float c2, const float* post_w,
+                                           const float* pre_w, void* h, float eps, int32_t T, int32_t W, const void* router_w, const float* router_bias,
+                                           int32_t n_router, int32_t top, int32_t* pair_expert, float* pair_weight, int32_t dtype, int64_t stream) {
+  StkSandwichArgs a;
+  a.x = x, a.p1 = p1, a.n1 = n1, a.pw = pw, a.c1 = c1, a.p2 = p2, a.c2 = c2, a.post_w = post_w, a.pre_w = pre_w, a.h = h, a.eps = eps, a.T = T, a.W = W;
+  a.router_w = router_w, a.router_bias = router_bias, a.n_router = n_router, a.top = top, a.pair_expert = pair_expert, a.pair_weight = pair_weight;
+  vra_stack_sandwich_norm(a, dtype, stream);
+}
