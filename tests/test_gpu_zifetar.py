@@ -94,7 +94,7 @@ ALONE = {
     "delta-one-group-conv1": [delta(heads=3, kv_heads=1, dim=8, vdim=40, conv=1)],
     "delta-wide": [delta(heads=2, kv_heads=2, dim=128, vdim=128, conv=3)],
     "retention": [retention()],
-    "retention-full-rotary": [retention(heads=2, dim=64, vdim=64, decay=(0.96875, 0.999), dims=64, base=1e6)],
+    "retention-full-rotary": [retention(heads=2, dim=64, vdim=48, decay=(0.97, 0.999), dims=64, base=2e5)],
     "retention-no-rotary": [retention(dims=0)],
     "attention-branch": [parallel(rs=0.0)],
     "attention-branch-plain-causal": [parallel(size=0, scaling=False, rs=0.0)],
@@ -354,12 +354,12 @@ def test_long_decoding(model):
 def test_long_prompt_in_one_step_and_in_portions():
     """a 1500-token prompt through heads of 64 / 128 channels (bf16 prompt steps of this size take the matrix-core attention and matrix
     kernels), whole and in three portions"""
-    cfg = config([dict(parallel(heads=8, kv_heads=2, dim=64, vdim=64, size=200, dims=64, r_heads=2, r_dim=32, r_vdim=32, scale=0.125), mlp=MOE),
+    cfg = config([dict(parallel(heads=4, kv_heads=2, dim=64, vdim=32, size=192, dims=32, r_heads=2, r_dim=32, r_vdim=64, scale=0.11), mlp=MOE),
                   dict(delta(heads=2, kv_heads=1, dim=64, vdim=64, conv=3), mlp=None),
                   dict(retention(heads=2, dim=128, vdim=64, decay=(0.99, 0.9995), dims=32), mlp=MOE)], width=128)
     tensors = zo.random_tensors(cfg, 23)
     toks = tokens_of(cfg, 1500, 8)
-    want = list(range(0, 1500, 47)) + [199, 200, 201, 1499]
+    want = list(range(0, 1500, 47)) + [191, 192, 193, 1499]
     want.sort()
     ref = zo.forward(cfg, tensors, toks)[want]
     for dt in (F32, BF16):
@@ -490,7 +490,7 @@ def run_masked_attention(L, q, positions, k, v, scale, chunk, dt, decode, r, BS=
 
 @pytest.mark.parametrize("dt", [F32, BF16], ids=["f32", "bf16"])
 @pytest.mark.parametrize("decode", [False, True], ids=["prompt", "decoded"])
-@pytest.mark.parametrize("chunk,dim,vdim", [(200, 32, 16), (64, 16, 8), (70, 64, 64), (1, 16, 8)])
+@pytest.mark.parametrize("chunk,dim,vdim", [(150, 32, 16), (64, 16, 8), (70, 64, 64), (1, 16, 8)])
 def test_block_mask_planted_key(dt, decode, chunk, dim, vdim):
     """one key stands out among 900 (its value is a marker).  A query in the key's own block of positions and not before it returns the
     marker — at the block's first and last position, across page borders; a query of the next block, or of the block before, or before
@@ -592,13 +592,13 @@ def test_seam_norms_and_router(dt, W, E, top):
     post, pre = (1 + 0.2 * r.standard_normal(W)).astype(np.float32), (1 + 0.2 * r.standard_normal(W)).astype(np.float32)
     rw = zo.bf16_round((r.standard_normal((E, W)) / math.sqrt(W)).astype(np.float32))
     rb = (0.3 * r.standard_normal(E)).astype(np.float32)
-    s = 0.6 * (pw[:, None] * p1).reshape(T, n1, W).sum(1).astype(np.float64) + 0.9 * p2
+    s = 0.75 * (pw[:, None] * p1).reshape(T, n1, W).sum(1).astype(np.float64) + 1.25 * p2
     x_ref = x + zo.rms(s, eps) * post
     h_ref = zo.rms(x_ref, eps) * pre
     z = h_ref @ rw.T.astype(np.float64) + rb
     xd, hd = raw(x, np.float32), empty(T * W * 4)
     pe, pwt = empty(T * top * 4), empty(T * top * 4)
-    L.vra_stack_op_sandwich_norm(xd.ptr, raw(p1, np.float32).ptr, n1, raw(pw, np.float32).ptr, 0.6, raw(p2, np.float32).ptr, 0.9, raw(post, np.float32).ptr,
+    L.vra_stack_op_sandwich_norm(xd.ptr, raw(p1, np.float32).ptr, n1, raw(pw, np.float32).ptr, 0.75, raw(p2, np.float32).ptr, 1.25, raw(post, np.float32).ptr,
                                  raw(pre, np.float32).ptr, hd.ptr, eps, T, W, to_dev(rw, dt).ptr, raw(rb, np.float32).ptr, E, top, pe.ptr, pwt.ptr, dt, 0)
     check()
     assert rel(xd.numpy(np.float32, (T, W)), x_ref) < 1e-6

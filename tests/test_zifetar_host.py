@@ -201,7 +201,7 @@ def test_decay_forms():
     w = zo.random_tensors(cfg, 3)
     # sigmoid(z)^(1 / tau) stays in (0, 1) and grows with tau
     z = np.array([-3.0, 0.0, 3.0])
-    a4, a16 = np.exp(np.log(zo.sigmoid(z)) / 4.0), np.exp(np.log(zo.sigmoid(z)) / 16.0)
-    assert np.all(a4 < a16) and np.all(a16 < 1.0) and np.isclose(a4[1], 0.5 ** 0.25)
+    a4, a9 = np.exp(np.log(zo.sigmoid(z)) / 4.0), np.exp(np.log(zo.sigmoid(z)) / 9.0)
+    assert np.all(a4 < a9) and np.all(a9 < 1.0) and np.isclose(a4[1], 0.5 ** 0.25)
     assert zo.forward(cfg, w, [1, 2, 3]).shape == (3, 50)
     assert np.isclose(zo.softplus(np.array([0.0]))[0], math.log(2.0)) and np.isclose(zo.softplus(np.array([50.0]))[0], 50.0)

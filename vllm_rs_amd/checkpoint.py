@@ -178,7 +178,7 @@ def parse_zifetar(cfg_json, dtype=None):
         mx, kind = layer["mixer"], layer.get("type")
         if kind == "channel_delta":
             f = dict(mixer="delta", heads=int(mx["heads"]), kv_heads=int(mx.get("kv_heads", mx["heads"])), dim=int(mx["dim"]),
-                     vdim=int(mx.get("vdim", mx["dim"])), conv=int(mx.get("conv", 1)), rank_a=int(mx.get("rank_a", 16)), rank_g=int(mx.get("rank_g", 16)))
+                     vdim=int(mx.get("vdim", mx["dim"])), conv=int(mx.get("conv", 1)), rank_a=int(mx.get("rank_a", 32)), rank_g=int(mx.get("rank_g", 32)))
         elif kind == "retention":
             f = dict(mixer="retention", heads=int(mx["heads"]), dim=int(mx["dim"]), vdim=int(mx.get("vdim", mx["dim"])),
                      decay=",".join(_num(d) for d in mx["decay"]))
@@ -189,7 +189,7 @@ def parse_zifetar(cfg_json, dtype=None):
                      vdim=int(le.get("vdim", le["dim"])), scale=_num(le["scale"]) if le.get("scale") is not None else _num(int(le["dim"]) ** -0.5),
                      chunk=int((le.get("mask") or {}).get("size", 0)), qk_norm=1, bias=1,
                      r_heads=int(ri["heads"]), r_dim=int(ri["dim"]), r_vdim=int(ri.get("vdim", ri["dim"])), tau=_num(ri["tau"]),
-                     rank_a=int(ri.get("rank_a", 16)), left_scale=_num(mx.get("left_scale", 1.0)), right_scale=_num(mx.get("right_scale", 1.0)))
+                     rank_a=int(ri.get("rank_a", 32)), left_scale=_num(mx.get("left_scale", 1.0)), right_scale=_num(mx.get("right_scale", 1.0)))
             f.update(rot_fields(le))
         else:
             raise ValueError(f"layer {i}: mixer type {kind!r} is not part of this design")

@@ -78,15 +78,15 @@ def gaperax_costs(cj):
 
 def zifetar_config(width, heads, kv_heads, dim, layers, vocab, experts, top, expert_ff, chunk, rank):
     """config.json dict of a Zifetar model: layers in the order parallel, delta rule, retention, ...; every layer a mixture of experts"""
-    rot = dict(base=5e5, dims=dim, scaling=dict(factor=8.0, low=1.0, high=4.0, original=8192))
+    rot = dict(base=2e5, dims=dim, scaling=dict(factor=4.0, low=1.0, high=8.0, original=4096))
     par = dict(left=dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim, scale=dim ** -0.5, mask=dict(size=chunk), rot=rot),
-               right=dict(heads=heads // 2, dim=dim, vdim=dim, tau=16.0, rank_a=rank), left_scale=0.6, right_scale=0.9)
+               right=dict(heads=heads // 2, dim=dim, vdim=dim, tau=8.0, rank_a=rank), left_scale=0.5, right_scale=1.0)
     dl = dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim, conv=4, rank_a=rank, rank_g=rank)
-    ret = dict(heads=heads, dim=dim, vdim=dim, decay=[1.0 - 2.0 ** (-5.0 - 5.0 * h / max(heads - 1, 1)) for h in range(heads)], rot=dict(base=1e6, dims=dim))
+    ret = dict(heads=heads, dim=dim, vdim=dim, decay=[1.0 - 2.0 ** (-5.0 - 5.0 * h / max(heads - 1, 1)) for h in range(heads)], rot=dict(base=1e5, dims=dim))
     mlp = dict(kind="moe", expert=dict(ff=expert_ff), router=dict(experts=experts, top=top))
     kinds = [("parallel", par), ("channel_delta", dl), ("retention", ret)]
     ls = [dict(type=kinds[i % 3][0], mixer=kinds[i % 3][1], mlp=mlp) for i in range(layers)]
-    return dict(architecture="Zifetar", width=width, vocab=vocab, norm=dict(eps=1e-6), embedding=dict(scale=width ** 0.5, bigram=dict(buckets=65521, mul_prev=31, mul_cur=7)),
+    return dict(architecture="Zifetar", width=width, vocab=vocab, norm=dict(eps=1e-6), embedding=dict(scale=width ** 0.5, bigram=dict(buckets=65521, mul_prev=257, mul_cur=3)),
                 layers=ls)
 
 
