@@ -355,6 +355,10 @@ bool StackModel::finalize_weights() {
       const int64_t ra = rows_of(p + "mix.a1", W), rg = rows_of(p + "mix.g1", W);
       if (ra < 1 || rg < 1) return error = "tensor " + p + "mix.a1 / g1: missing or of another width", false;
       L.rank_a = (int)ra, L.rank_g = (int)rg;
+      {  // the taps of the short convolutions are the columns of their tensors
+        auto it = staged_.find(p + "mix.q.conv");
+        if (it != staged_.end() && it->second.shape.size() == 2 && it->second.shape[1] >= 1) L.conv = (int)it->second.shape[1];
+      }
       const HostTensor *q, *k, *v, *bw, *a1, *g1, *a2, *g2, *cq, *ck, *cv, *al;
       if (!need(p + "mix.q", nk, W, &q) || !need(p + "mix.k", nk, W, &k) || !need(p + "mix.v", nv, W, &v) || !need(p + "mix.b", H, W, &bw) ||
           !need(p + "mix.a1", ra, W, &a1) || !need(p + "mix.g1", rg, W, &g1) || !need(p + "mix.a2", (int64_t)H * L.dim, ra, &a2) ||
