@@ -208,7 +208,65 @@ def parse_zifetar(cfg_json, dtype=None):
                 rms_norm_eps=float(norm.get("eps", 1e-6)), rope_theta=10000.0, dtype=dt, quant_method=None, spec="\n".join(lines) + "\n")
 
 
-STACK_ARCHS = {"Ditilix": parse_ditilix, "Gaperax": parse_gaperax, "Zifetar": parse_zifetar}
+def parse_sudosun(cfg_json, dtype=None):
+    """Sudosun config.json -> cfg dict with arch "stack": sandwich blocks whose four norms are Dynamic Tanh, a plain embedding whose table is
+    also the head, per layer one of three mixers that carry a state per sequence (a gated delta rule with one decay per head, lightning
+    attention with constant decays, softmax attention under a sliding window with a sink beside a real-gated diagonal recurrence) and a
+    feed-forward that is dense (clamped gated form) or a mixture of experts (softmax over all router outputs, a correction for the choice,
+    expert groups, identity experts).  Every size and constant comes from the config; the taps of the convolutions come from their tensors."""
+    td = dtype or cfg_json.get("torch_dtype", "bfloat16")
+    dt = {"bfloat16": BF16, "bf16": BF16, "float32": F32, "f32": F32, BF16: BF16, F32: F32}.get(td)
+    if dt is None:
+        raise ValueError(f"dtype {td!r}: a layer stack runs in bfloat16 or float32")
+    norm = cfg_json.get("norm") or {}
+    width, vocab, layers = int(cfg_json["width"]), int(cfg_json["vocab"]), cfg_json["layers"]
+    lines = ["stack width=%d vocab=%d eps=%s block=sandwich norm=dyt pos=none tie_head=1 logit_scale=%s" % (
+        width, vocab, _num(norm.get("eps", 1e-6)), _num(cfg_json.get("logit_scale", 1.0)))]
+    heads = kv_heads = dim = 1
+    for i, layer in enumerate(layers):
+        mx, kind = layer["mixer"], layer.get("type")
+        if kind == "delta":
+            f = dict(mixer="delta", lowrank=0, heads=int(mx["heads"]), kv_heads=int(mx.get("kv_heads", mx["heads"])), dim=int(mx["dim"]),
+                     vdim=int(mx.get("vdim", mx["dim"])), conv=int(mx.get("conv", 1)))
+        elif kind == "lightning":
+            f = dict(mixer="lightning", heads=int(mx["heads"]), dim=int(mx["dim"]), vdim=int(mx.get("vdim", mx["dim"])),
+                     decay=",".join(_num(d) for d in mx["decay"]))
+        elif kind == "parallel":
+            le, ri = mx["left"], mx["right"]
+            rot = le.get("rot") or {}
+            f = dict(mixer="parallel", right="rglru", heads=int(le["heads"]), kv_heads=int(le.get("kv_heads", le["heads"])), dim=int(le["dim"]),
+                     vdim=int(le.get("vdim", le["dim"])), scale=_num(le["scale"]) if le.get("scale") is not None else _num(int(le["dim"]) ** -0.5),
+                     window=int((le.get("mask") or {}).get("size", 0)), qk_norm=1, bias=1, sink=1, head_temp=1, head_gate=1, branch_norm=1,
+                     rot_layout="pairs", rot_dims=int(rot.get("dims", 0)), rot_base=_num(rot.get("base", 10000.0)),
+                     r_width=int(ri["width"]), r_blocks=int(ri.get("blocks", 1)), r_conv=int(ri.get("conv", 1)), left_scale=_num(0.5), right_scale=_num(0.5))
+            sc = rot.get("scaling")
+            if sc:
+                f.update(yarn_factor=_num(sc["factor"]), yarn_original=_num(sc["original"]), yarn_fast=_num(sc.get("fast", 32.0)),
+                         yarn_slow=_num(sc.get("slow", 1.0)))
+        else:
+            raise ValueError(f"layer {i}: mixer type {kind!r} is not part of this design")
+        mlp = layer.get("mlp")
+        if not mlp:
+            f.update(mlp="none")
+        elif mlp["kind"] == "dense":
+            f.update(mlp="clamped", ff=int(mlp["ff"]), limit=_num(mlp["limit"]))
+        elif mlp["kind"] == "moe":
+            r = mlp["router"]
+            f.update(mlp="moe", ff=int(mlp["expert"]["ff"]), experts=int(r["experts"]), top=int(r.get("top", 1)), router="softmax_all", act="silu",
+                     identity=int(r.get("identity", 0)))
+            g = r.get("groups")
+            if g:
+                f.update(groups=int(g["count"]), keep=int(g["keep"]))
+        else:
+            raise ValueError(f"layer {i}: feed-forward kind {mlp['kind']!r} is not part of this design")
+        lines.append("layer " + " ".join(f"{k}={v}" for k, v in f.items()))
+        heads, kv_heads, dim = max(heads, f["heads"]), max(kv_heads, f.get("kv_heads", f["heads"])), max(dim, f["dim"], f["vdim"])
+    return dict(arch="stack", design="Sudosun", hidden_size=width, vocab_size=vocab, num_layers=len(layers), num_heads=heads, num_kv_heads=kv_heads,
+                head_dim=dim, intermediate_size=0, max_position_embeddings=int(cfg_json.get("max_position_embeddings", 1 << 20)),
+                rms_norm_eps=float(norm.get("eps", 1e-6)), rope_theta=10000.0, dtype=dt, quant_method=None, spec="\n".join(lines) + "\n")
+
+
+STACK_ARCHS = {"Ditilix": parse_ditilix, "Gaperax": parse_gaperax, "Zifetar": parse_zifetar, "Sudosun": parse_sudosun}
 
 
 def parse_config(cfg_json, dtype=None):

@@ -36,6 +36,7 @@ struct StkGemmArgs {
   // (element counts; a column offset per head turns one launch into a product per head)
   int batch = 1;
   int64_t a_batch_stride = 0, w_batch_stride = 0, out_batch_stride = 0;
+  int64_t bias_batch_stride = 0;  // elements between the bias rows of two products of a batch
 };
 void vra_stack_gemm(const StkGemmArgs& g, int dtype, int64_t stream);
 // rows per granule the grouped launches of an M-row problem over `groups` groups want (16 or 64)
@@ -105,6 +106,10 @@ struct StkAttnArgs {
                                 // part] per token: keys are the whole row, values its first columns (vc = kc, v_ld = k_ld)
   int chunk = 0;                // > 0: key j is visible only if it lies in the query's own block of `chunk` positions,
                                 // floor(j / chunk) = floor(p_i / chunk); blocks count from position 0 of the sequence
+  int window = 0;               // > 0: key j is visible only if p_i - j < window (the query's own position and the window - 1 before it)
+  const float* head_scale = nullptr;  // f32 [H]: head h's scores are also multiplied by head_scale[h] (the sink is not)
+  const float* gate = nullptr;  // f32 [T, gate_ld], column h: head h's output row is multiplied by sigmoid(gate[t, h])
+  int gate_ld = 0;
 };
 void vra_stack_attention(const StkAttnArgs& a, int dtype, int64_t stream);
 
@@ -215,11 +220,18 @@ struct StkEmbedPairArgs {
 void vra_stack_embed_pair(const StkEmbedPairArgs& a, int dtype, int64_t stream);
 
 // The seam between two sub-blocks of a sandwich-norm stack, one launch:
-//   s = c1 * sum_{j < n1} pw[t * n1 + j] * p1[(t * n1 + j), :]  +  c2 * p2[t, :]      (pw null: weights 1; p2 null: no second part)
+//   s = c1 * sum_{j < n1} pw[t * n1 + j] * p1[(t * n1 + j), :]  +  c2 * p2w[t] * p2[t, :]   (pw, p2w null: weights 1; p2 null: no second part;
+//                                                                                       pe: pairs with pe[t * n1 + j] < 0 have no row and are left out)
+//   with p1_norm_w / p2_norm_w (n1 = 1): each part is first divided by its root mean square over the row and multiplied by that weight
 //   x[t] += N(s; post_w)                                                              (post_w null: nothing is added)
-//   h[t]  = N(x[t]; pre_w)  in dtype                                                  (pre_w null: no h)
-// and, with router_w ([n_router, W] in dtype): z = router_w . h + router_bias on the unrounded h, the `top` largest (ties: the lower
-// index) -> pair_expert / pair_weight [T, top], weights = softmax over the chosen logits.  All f32.
+//   h[t]  = N(x[t]; pre_w)  in dtype                                                  (pre_w null: no h);  h32: also the unrounded h (f32)
+// N is an RMS norm with a weight, or (dyt) Dynamic Tanh  tanh(alpha v) w + b  with the slopes post_alpha / pre_alpha and offsets post_b / pre_b.
+// With router_w ([n_router, W] in dtype): z = router_w . h + router_bias on the unrounded h, the `top` largest (ties: the lower
+// index) -> pair_expert / pair_weight [T, top].  router_kind 0: weights = softmax over the chosen logits.  router_kind 1: scores =
+// softmax over all n_router logits; the choice goes by score + router_bias (a correction that the weights do not carry) among the experts of
+// the `keep` groups (of n_groups equal groups of neighbours) whose largest corrected score is largest; weights = the chosen scores as they
+// are; the last n_identity router outputs are experts without tensors that hand their input back: their pairs get expert -1 and their
+// weights are summed into id_weight[t].  All f32.
 struct StkSandwichArgs {
   float* x = nullptr;
   const float* p1 = nullptr;
@@ -238,6 +250,17 @@ struct StkSandwichArgs {
   int n_router = 0, top = 0;
   int* pair_expert = nullptr;
   float* pair_weight = nullptr;
+  int dyt = 0;
+  const float* post_b = nullptr;
+  const float* pre_b = nullptr;
+  float post_alpha = 1.f, pre_alpha = 1.f;
+  const float* p1_norm_w = nullptr;
+  const float* p2_norm_w = nullptr;
+  const int* pe = nullptr;
+  const float* p2w = nullptr;
+  float* h32 = nullptr;
+  int router_kind = 0, n_groups = 0, keep = 0, n_identity = 0;
+  float* id_weight = nullptr;
 };
 void vra_stack_sandwich_norm(const StkSandwichArgs& a, int dtype, int64_t stream);
 
@@ -264,6 +287,7 @@ struct StkHeadPrepArgs {
   const int64_t* slots = nullptr;
   int out_f32 = 0;
   int T = 0;
+  int rot_pairs_layout = 0;  // 1: dimension 2i pairs with 2i + 1 (neighbours) instead of i with i + rot.pairs
 };
 void vra_stack_head_prep(const StkHeadPrepArgs& a, int dtype, int64_t stream);
 
@@ -283,6 +307,7 @@ struct StkDeltaPrepArgs {
   const float* rate = nullptr;     // [H]
   const float* dt_bias = nullptr;  // [H * dim]
   float q_scale = 1.f;
+  int decay_dim = 0;               // decays a head: 0 = one per key channel (raw2 / dt_bias / decay_out carry H * dim), 1 = one per head (H)
   float* qkv_out = nullptr;
   float* beta_out = nullptr;
   float* decay_out = nullptr;
@@ -311,6 +336,8 @@ struct StkScanArgs {
   int ldv = 0;
   const float* decay = nullptr;
   int ldd = 0;
+  int decay_per_head = 0;  // 1: decay [T, ldd] holds ONE decay per head and token (column h) instead of one per key channel
+  int act_silu = 0;        // 1: q, k and v pass silu on their way in (constant decays per head only)
   const float* head_decay = nullptr;
   const float* beta = nullptr;
   int ldb = 0;
@@ -329,3 +356,51 @@ void vra_stack_linear_scan(const StkScanArgs& a, int64_t stream);
 // gate_act 1: silu, 2: sigmoid);  o f32 [T, H * vdim], out in dtype
 void vra_stack_head_norm_gate(const float* o, const float* w, const float* gate, int gate_ld, int gate_act, float eps, void* out, int T, int H, int vdim,
                               int dtype, int64_t stream);
+
+// ---------------------------------------------------------------------------------------------------------------------------------------
+// A short causal convolution over time per channel with its state, and a gated diagonal linear recurrence (stack_recurrent.hip)
+
+// y[t, c] = act(bias[c] + sum_j w[c, j] x[t - (taps - 1 - j), c])   (x f32 [T, ld]; w f32 [C, taps], last column = the current token; the inputs
+// before a step's first row come from conv_state [slots, taps - 1, C], zeros for a sequence that starts; act 0 none, 1 silu; bias may be null).
+// vra_stack_conv_rows_update then moves the state on (the last taps - 1 inputs of every sequence).
+struct StkConvArgs {
+  const float* x = nullptr;
+  int ld = 0, C = 0, taps = 1;
+  const float* w = nullptr;
+  const float* bias = nullptr;
+  float* conv_state = nullptr;
+  int act = 0;
+  float* y = nullptr;
+  int ldy = 0;
+  const int64_t* positions = nullptr;
+  const uint32_t* cu_q = nullptr;
+  const int32_t* state_slots = nullptr;
+  int T = 0, B = 0;
+};
+void vra_stack_conv_rows(const StkConvArgs& a, int64_t stream);
+void vra_stack_conv_rows_update(const StkConvArgs& a, int64_t stream);
+
+// Real-gated diagonal recurrence over a sequence's tokens, one state value per channel (f32 [slots, C]):
+//   r = sigmoid(gr[t, c]), i = sigmoid(gi[t, c]), a = exp(-rate * r * softplus(lam[c])),  S <- a S + sqrt(1 - a^2) (i u[t, c]),
+//   out[t, c] = S * gelu_tanh(y[t, c])  in dtype.
+// Tokens run in order; a sequence whose first row stands at position 0 starts from S = 0.
+struct StkGatedScanArgs {
+  const float* u = nullptr;
+  int ldu = 0;
+  const float* gr = nullptr;
+  const float* gi = nullptr;
+  int ldg = 0;
+  int block = 0;  // > 0: the gates come in blocks — channel c's logits stand at column (c / block) * 2 * block + c % block of gr and gi
+  const float* y = nullptr;
+  int ldy = 0;
+  const float* lam = nullptr;
+  float rate = 8.f;
+  float* state = nullptr;
+  const int32_t* state_slots = nullptr;
+  const int64_t* positions = nullptr;
+  const uint32_t* cu_q = nullptr;
+  void* out = nullptr;
+  int ldo = 0;
+  int B = 0, C = 0;
+};
+void vra_stack_gated_scan(const StkGatedScanArgs& a, int dtype, int64_t stream);

@@ -206,7 +206,7 @@ __global__ __launch_bounds__(256) void stk_gemm_simple_kernel(StkGemmArgs g) {
     for (int j = 0; j < 4; j++) {
       const int n = n0 + tx * 4 + j;
       if (n >= g.N) continue;
-      const float v = acc[i][j] * g.alpha + (g.bias ? g.bias[n] : 0.f);
+      const float v = acc[i][j] * g.alpha + (g.bias ? g.bias[(int64_t)blockIdx.z * g.bias_batch_stride + n] : 0.f);
       if (g.out_f32) ((float*)g.out)[ob + (int64_t)orow * g.ldo + n] = v;
       else El<T>::st((T*)g.out + ob + (int64_t)orow * g.ldo + n, v);
     }
@@ -315,7 +315,7 @@ __global__ __launch_bounds__(64 * WM * WN) void stk_gemm_mfma_kernel(StkGemmArgs
         for (int j = 0; j < 4; j++) {
           const int n = n_base + nt * 16 + oct * 4 + j;
           if (n >= g.N) continue;
-          const float v = acc[mt][nt][j] * g.alpha + (g.bias ? g.bias[n] : 0.f);
+          const float v = acc[mt][nt][j] * g.alpha + (g.bias ? g.bias[(int64_t)blockIdx.z * g.bias_batch_stride + n] : 0.f);
           if (g.out_f32) ((float*)g.out)[ob + (int64_t)orow * g.ldo + n] = v;
           else ((uint16_t*)g.out)[ob + (int64_t)orow * g.ldo + n] = BF16::from_f32(v);
         }
@@ -401,7 +401,7 @@ __global__ __launch_bounds__(512) void stk_gemm_mfma_small_kernel(StkGemmArgs g)
   } else {
     const int n = n_base + c;
     if (n >= g.N) return;
-    const float v = total(c) * g.alpha + (g.bias ? g.bias[n] : 0.f);
+    const float v = total(c) * g.alpha + (g.bias ? g.bias[(int64_t)blockIdx.z * g.bias_batch_stride + n] : 0.f);
     if (g.out_f32) ((float*)g.out)[ob + (int64_t)orow * g.ldo + n] = v;
     else ((uint16_t*)g.out)[ob + (int64_t)orow * g.ldo + n] = BF16::from_f32(v);
   }
@@ -534,7 +534,10 @@ __global__ __launch_bounds__(256) void stk_attn_prefill_kernel(StkAttnArgs a) {
   }
   int64_t pq[4], plo[4];
   int64_t pmax = -1, lo_min = INT64_MAX;
-  auto block_start = [&](int64_t p) { return a.chunk > 0 ? p / a.chunk * a.chunk : (int64_t)0; };  // first key a query at p may see
+  auto block_start = [&](int64_t p) {  // first key a query at p may see
+    const int64_t lo = a.chunk > 0 ? p / a.chunk * a.chunk : (int64_t)0;
+    return a.window > 0 ? max(lo, p - a.window + 1) : lo;
+  };
   for (int i = 0; i < 4; i++) {
     const int r = wave * 4 + i;
     pq[i] = r < nq ? a.positions[t0 + r] : -1;
@@ -553,6 +556,7 @@ __global__ __launch_bounds__(256) void stk_attn_prefill_kernel(StkAttnArgs a) {
   const T* vc = (const T*)a.vc;
   const uint32_t* bt = a.block_tables + (size_t)b * a.max_blocks;
   const int kdim = a.k_ld ? a.k_ld : a.G * dim, vd_all = a.v_ld ? a.v_ld : a.G * vdim;
+  const float hscale = a.head_scale ? a.scale * a.head_scale[h] : a.scale;
   for (int kt0 = kt_begin; kt0 < n_keys; kt0 += KT) {
     __syncthreads();
     for (int i = tid; i < KT * dim; i += 256) {
@@ -580,7 +584,7 @@ __global__ __launch_bounds__(256) void stk_attn_prefill_kernel(StkAttnArgs a) {
       if (lane < KT && pq[i] >= 0 && kt0 + lane <= pq[i] && kt0 + lane >= plo[i] && kt0 + lane < n_keys) {
         float d0 = 0.f;
         for (int d = 0; d < dim; d++) d0 = fmaf(qs[r * dim + d], ks[lane * kld + d], d0);
-        s = cap_score(d0 * a.scale, a.softcap);
+        s = cap_score(d0 * hscale, a.softcap);
       }
       const float mn = fmaxf(m[i], wave_max(s));
       float p = 0.f, corr = 1.f;
@@ -608,7 +612,8 @@ __global__ __launch_bounds__(256) void stk_attn_prefill_kernel(StkAttnArgs a) {
   for (int i = 0; i < 4; i++) {
     const int r = wave * 4 + i;
     if (r >= nq) continue;
-    const float inv = l[i] > 0.f ? 1.f / l[i] : 0.f;
+    float inv = l[i] > 0.f ? 1.f / l[i] : 0.f;
+    if (a.gate) inv *= sigmoidf_(a.gate[(size_t)(t0 + r) * a.gate_ld + h]);
     for (int rr = 0; rr < 4; rr++) {
       const int d = lane + 64 * rr;
       if (d < vdim) El<T>::st(out + (size_t)(t0 + r) * a.H * vdim + h * vdim + d, acc[i][rr] * inv);
@@ -648,12 +653,13 @@ __global__ __launch_bounds__(256) void stk_attn_prefill_mfma_kernel(StkAttnArgs 
     const u32x4 v = *(const u32x4*)(q + (size_t)(ok ? tq : q0) * a.ldq + h * dim + (ok ? ch : 0));
     qf[c] = ok ? v : zero4;
   }
-  const float sc = a.scale * q_temperature(pq < 0 ? 0 : pq, a.temp_coef, a.temp_every);
+  const float sc = a.scale * q_temperature(pq < 0 ? 0 : pq, a.temp_coef, a.temp_every) * (a.head_scale ? a.head_scale[h] : 1.f);
   // keys this workgroup needs: up to the largest position of its rows
   int64_t pmax = pq;
   for (int o = 32; o > 0; o >>= 1) pmax = max(pmax, (int64_t)__shfl_xor((long long)pmax, o, 64));
   // block mask: this row sees the keys from key_lo on; the workgroup's tiles start at the tile of its smallest key_lo
-  const int64_t key_lo = a.chunk > 0 && pq >= 0 ? pq / a.chunk * a.chunk : 0;
+  int64_t key_lo = a.chunk > 0 && pq >= 0 ? pq / a.chunk * a.chunk : 0;
+  if (a.window > 0 && pq >= 0) key_lo = max(key_lo, pq - a.window + 1);
   int64_t lmin = pq >= 0 ? key_lo : INT64_MAX;
   for (int o = 32; o > 0; o >>= 1) lmin = min(lmin, (int64_t)__shfl_xor((long long)lmin, o, 64));
   __shared__ long long wmax[4], wmin[4];
@@ -802,7 +808,8 @@ __global__ __launch_bounds__(256) void stk_attn_prefill_mfma_kernel(StkAttnArgs 
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
   if (!qv) return;
-  const float inv = l > 0.f ? 1.f / l : 0.f;
+  float inv = l > 0.f ? 1.f / l : 0.f;
+  if (a.gate) inv *= sigmoidf_(a.gate[(size_t)tq * a.gate_ld + h]);
   uint16_t* out = (uint16_t*)a.out + (size_t)tq * a.H * vdim + h * vdim;
   for (int t = 0; t < VT; t++)
     for (int j = 0; j < 4; j++) {
@@ -868,14 +875,16 @@ __global__ __launch_bounds__(64 * STK_DW) void stk_attn_decode_kernel(StkAttnArg
   float vacc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   // block mask: the keys from key_lo on; tiles stay aligned to absolute positions (the first one may begin below key_lo: those keys
   // count with weight 0)
-  const int key_lo = a.chunk > 0 ? (int)(p / a.chunk * a.chunk) : 0;
+  int key_lo = a.chunk > 0 ? (int)(p / a.chunk * a.chunk) : 0;
+  if (a.window > 0) key_lo = max(key_lo, (int)(p - a.window + 1));
+  const float hscale = a.head_scale ? a.scale * a.head_scale[h] : a.scale;
   for (int kt0 = key_lo / 64 * 64 + wave * 64; kt0 < n_keys; kt0 += STK_DW * 64) {
     const int key = kt0 + lane;
     float s = -INFINITY;
     if (key < n_keys) {
       const int64_t slot = (int64_t)bt[key / a.BS] * a.BS + key % a.BS;
       ss[wave * 64 + lane] = (int)slot;
-      if (key >= key_lo) s = cap_score(stk_dot_row<T>(qs, kc + slot * kdim + g * dim, dim) * a.scale, a.softcap);
+      if (key >= key_lo) s = cap_score(stk_dot_row<T>(qs, kc + slot * kdim + g * dim, dim) * hscale, a.softcap);
     }
     const float mn = fmaxf(m, wave_max(s));  // (the tile's first key exists: mn is finite)
     const float pj = s > -INFINITY ? expf(s - mn) : 0.f;
@@ -937,6 +946,7 @@ __global__ __launch_bounds__(64 * STK_DW) void stk_attn_decode_kernel(StkAttnArg
   float M = ms[0];
   for (int w = 1; w < STK_DW; w++) M = fmaxf(M, ms[w]);
   T* out = (T*)a.out + (size_t)b * a.H * vdim + h * vdim;
+  const float og = a.gate ? sigmoidf_(a.gate[(size_t)b * a.gate_ld + h]) : 1.f;
   for (int d = tid; d < vdim; d += 64 * STK_DW) {
     float L = 0.f, o = 0.f;
     for (int w = 0; w < STK_DW; w++) {
@@ -944,7 +954,7 @@ __global__ __launch_bounds__(64 * STK_DW) void stk_attn_decode_kernel(StkAttnArg
       L += ms[STK_DW + w] * c;
       o += os[w * vdim + d] * c;
     }
-    El<T>::st(out + d, L > 0.f ? o / L : 0.f);
+    El<T>::st(out + d, L > 0.f ? o / L * og : 0.f);
   }
 }
 

@@ -73,41 +73,81 @@ __global__ __launch_bounds__(256) void stk_sandwich_kernel(StkSandwichArgs a) {
   extern __shared__ float lds[];
   __shared__ float red[4];
   float* xs = lds;             // [W]
-  float* zs = lds + a.W;       // [n_router]
+  float* zs = lds + a.W;       // [n_router] logits / corrected scores, [n_router] scores, [n_groups] group scores
   const int t = blockIdx.x, W = a.W, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   float* x = a.x + (size_t)t * W;
   if (a.post_w) {
+    // a branch with a norm of its own: its row's root mean square first (f32, the same order of sums as every norm here)
+    float r1 = 1.f, r2 = 1.f;
+    if (a.p1_norm_w) {
+      float q = 0.f;
+      for (int c = tid; c < W; c += 256) {
+        const float v = a.p1[(size_t)t * W + c];
+        q = fmaf(v, v, q);
+      }
+      r1 = 1.f / sqrtf(block_sum_256(q, red) / (float)W + a.eps);
+    }
+    if (a.p2 && a.p2_norm_w) {
+      float q = 0.f;
+      for (int c = tid; c < W; c += 256) {
+        const float v = a.p2[(size_t)t * W + c];
+        q = fmaf(v, v, q);
+      }
+      r2 = 1.f / sqrtf(block_sum_256(q, red) / (float)W + a.eps);
+    }
+    const float w2 = a.p2w ? a.p2w[t] : 1.f;
     float s = 0.f;
     for (int c = tid; c < W; c += 256) {
       float v = 0.f;
-      for (int j = 0; j < a.n1; j++) {
-        const size_t r = (size_t)t * a.n1 + j;
-        const float pv = a.p1[r * W + c];
-        v = a.pw ? fmaf(a.pw[r], pv, v) : v + pv;
+      if (a.p1_norm_w) {
+        v = a.p1[(size_t)t * W + c] * r1 * a.p1_norm_w[c];
+      } else {
+        for (int j = 0; j < a.n1; j++) {
+          const size_t r = (size_t)t * a.n1 + j;
+          if (a.pe && a.pe[r] < 0) continue;
+          const float pv = a.p1[r * W + c];
+          v = a.pw ? fmaf(a.pw[r], pv, v) : v + pv;
+        }
       }
       v *= a.c1;
-      if (a.p2) v = fmaf(a.c2, a.p2[(size_t)t * W + c], v);
+      if (a.p2) {
+        float v2 = a.p2[(size_t)t * W + c];
+        if (a.p2_norm_w) v2 = v2 * r2 * a.p2_norm_w[c];
+        v = fmaf(a.c2 * w2, v2, v);
+      }
       xs[c] = v;
       s = fmaf(v, v, s);
     }
-    const float r = 1.f / sqrtf(block_sum_256(s, red) / (float)W + a.eps);
-    for (int c = tid; c < W; c += 256) {
-      const float v = x[c] + xs[c] * r * a.post_w[c];
-      x[c] = v;
-      xs[c] = v;
+    if (a.dyt) {
+      for (int c = tid; c < W; c += 256) {
+        const float v = x[c] + (tanhf(a.post_alpha * xs[c]) * a.post_w[c] + a.post_b[c]);
+        x[c] = v;
+        xs[c] = v;
+      }
+    } else {
+      const float r = 1.f / sqrtf(block_sum_256(s, red) / (float)W + a.eps);
+      for (int c = tid; c < W; c += 256) {
+        const float v = x[c] + xs[c] * r * a.post_w[c];
+        x[c] = v;
+        xs[c] = v;
+      }
     }
   } else {
     for (int c = tid; c < W; c += 256) xs[c] = x[c];
   }
   if (!a.pre_w) return;
-  float s = 0.f;
-  for (int c = tid; c < W; c += 256) s = fmaf(xs[c], xs[c], s);
-  const float r = 1.f / sqrtf(block_sum_256(s, red) / (float)W + a.eps);
+  float r = 1.f;
+  if (!a.dyt) {
+    float s = 0.f;
+    for (int c = tid; c < W; c += 256) s = fmaf(xs[c], xs[c], s);
+    r = 1.f / sqrtf(block_sum_256(s, red) / (float)W + a.eps);
+  }
   T* h = (T*)a.h + (size_t)t * W;
   for (int c = tid; c < W; c += 256) {
-    const float v = xs[c] * r * a.pre_w[c];
+    const float v = a.dyt ? tanhf(a.pre_alpha * xs[c]) * a.pre_w[c] + a.pre_b[c] : xs[c] * r * a.pre_w[c];
     xs[c] = v;
     El<T>::st(h + c, v);
+    if (a.h32) a.h32[(size_t)t * W + c] = v;
   }
   if (!a.router_w) return;
   __syncthreads();
@@ -126,15 +166,17 @@ __global__ __launch_bounds__(256) void stk_sandwich_kernel(StkSandwichArgs a) {
       for (int c = lane; c < W; c += 64) z = fmaf(xs[c], El<T>::ld(rw + (size_t)e * W + c), z);
     }
     z = wave_sum(z);
-    if (lane == 0) zs[e] = z + (a.router_bias ? a.router_bias[e] : 0.f);
+    if (lane == 0) zs[e] = z + (a.router_kind == 0 && a.router_bias ? a.router_bias[e] : 0.f);
   }
   __syncthreads();
-  if (tid == 0) {  // the `top` largest in turn (ties: the lower index); a picked logit leaves the list
+  if (tid != 0) return;
+  const int n = a.n_router;
+  if (a.router_kind == 0) {  // the `top` largest in turn (ties: the lower index); a picked logit leaves the list
     float zmax = 0.f, sum = 0.f;
     for (int j = 0; j < a.top; j++) {
       int best = 0;
       float bz = zs[0];
-      for (int e = 1; e < a.n_router; e++)
+      for (int e = 1; e < n; e++)
         if (zs[e] > bz) best = e, bz = zs[e];
       zs[best] = -INFINITY;
       if (j == 0) zmax = bz;  // (the first pick is the largest logit)
@@ -145,7 +187,45 @@ __global__ __launch_bounds__(256) void stk_sandwich_kernel(StkSandwichArgs a) {
     }
     const float inv = 1.f / sum;
     for (int j = 0; j < a.top; j++) a.pair_weight[(size_t)t * a.top + j] *= inv;
+    return;
   }
+  // scores over all outputs; corrected scores choose, restricted to the best groups; the plain scores weigh
+  float* sc = zs + n;        // [n] scores
+  float* gs = zs + 2 * n;    // [n_groups]
+  float zmax = zs[0], sum = 0.f;
+  for (int e = 1; e < n; e++) zmax = fmaxf(zmax, zs[e]);
+  for (int e = 0; e < n; e++) sc[e] = expf(zs[e] - zmax), sum += sc[e];
+  const float inv = 1.f / sum;
+  for (int e = 0; e < n; e++) sc[e] *= inv, zs[e] = sc[e] + (a.router_bias ? a.router_bias[e] : 0.f);
+  if (a.n_groups > 1 && a.keep < a.n_groups) {
+    const int per = n / a.n_groups;
+    for (int g = 0; g < a.n_groups; g++) {
+      float b = zs[g * per];
+      for (int e = 1; e < per; e++) b = fmaxf(b, zs[g * per + e]);
+      gs[g] = b;
+    }
+    for (int g = 0; g < a.n_groups; g++) {  // a group stays if fewer than `keep` groups come before it (larger score, or equal and lower index)
+      int before = 0;
+      for (int o = 0; o < a.n_groups; o++) before += (gs[o] > gs[g] || (gs[o] == gs[g] && o < g)) ? 1 : 0;
+      if (before >= a.keep)
+        for (int e = 0; e < per; e++) zs[g * per + e] = -INFINITY;
+    }
+  }
+  float idw = 0.f;
+  const int n_real = n - a.n_identity;
+  for (int j = 0; j < a.top; j++) {
+    int best = -1;
+    float bz = -INFINITY;
+    for (int e = 0; e < n; e++)
+      if (sc[e] >= 0.f && (best < 0 || zs[e] > bz)) best = e, bz = zs[e];
+    const float w = sc[best];
+    sc[best] = -1.f;  // (picked: out of the list)
+    const bool ident = best >= n_real;
+    a.pair_expert[(size_t)t * a.top + j] = ident ? -1 : best;
+    a.pair_weight[(size_t)t * a.top + j] = w;
+    if (ident) idw += w;
+  }
+  if (a.id_weight) a.id_weight[t] = idw;
 }
 
 // ------------------------------------------------------------------------------------------------ per-head norm, rotary, cache rows
@@ -173,11 +253,13 @@ __global__ __launch_bounds__(256) void stk_head_prep_kernel(StkHeadPrepArgs a) {
     for (int c = lane; c < dim; c += 64) {
       float v = nw ? src[c] * r * nw[c] : src[c];
       if (c < 2 * rp) {
-        const int i = c < rp ? c : c - rp, oc = c < rp ? c + rp : c - rp;
+        const bool first = a.rot_pairs_layout ? (c & 1) == 0 : c < rp;
+        const int i = a.rot_pairs_layout ? c >> 1 : (c < rp ? c : c - rp);
+        const int oc = a.rot_pairs_layout ? c ^ 1 : (c < rp ? c + rp : c - rp);
         const float o = nw ? src[oc] * r * nw[oc] : src[oc];
         float cs, sn;
         rot_cos_sin(a.rot, i, p, &cs, &sn);
-        v = c < rp ? v * cs - o * sn : v * cs + o * sn;
+        v = first ? v * cs - o * sn : v * cs + o * sn;
       }
       El<TO>::st(dst + c, v * sc);
     }
@@ -232,8 +314,9 @@ __global__ __launch_bounds__(256) void stk_delta_prep_kernel(StkDeltaPrepArgs a)
   }
   for (int c = tid; c < H * vdim; c += 256) out[2 * nqk + c] = ys[2 * nqk + c];
   for (int h = tid; h < H; h += 256) a.beta_out[(size_t)t * H + h] = sigmoidf_(a.raw[(size_t)t * a.ld + C + h]);
-  for (int c = tid; c < H * dim; c += 256)
-    a.decay_out[(size_t)t * H * dim + c] = expf(-a.rate[c / dim] * softplusf_(a.raw2[(size_t)t * a.ld2 + c] + a.dt_bias[c]));
+  const int dd = a.decay_dim == 1 ? 1 : dim;
+  for (int c = tid; c < H * dd; c += 256)
+    a.decay_out[(size_t)t * H * dd + c] = expf(-a.rate[c / dd] * softplusf_(a.raw2[(size_t)t * a.ld2 + c] + a.dt_bias[c]));
 }
 
 // the last taps - 1 inputs of every sequence of the step -> its slot (after the step's rows have read what the slot held)
@@ -287,7 +370,8 @@ __device__ __forceinline__ float group_sum(float v) {
 
 // P, the presence of per-row decays and of the delta rule are template parameters: the 16 tokens of a tile are one straight line of code, so
 // the LDS reads of the tokens ahead are in flight while a token's sums run.
-template <int R, int P, bool DECAY, bool BETA>
+// DECAY 0: one constant per head; 1: one per row and key channel; 2: one per row and head.  ACT: q, k, v pass silu on their way into LDS.
+template <int R, int P, int DECAY, bool BETA, bool ACT>
 __global__ __launch_bounds__(256) void stk_linear_scan_kernel(StkScanArgs a) {
   constexpr int TT = 16, NL = 4;     // tokens a tile; 16-byte loads a thread and array for one tile (TT * dimP / 4 / 256, dimP <= 256)
   extern __shared__ __attribute__((aligned(16))) float lds[];
@@ -298,6 +382,7 @@ __global__ __launch_bounds__(256) void stk_linear_scan_kernel(StkScanArgs a) {
   float* ds = qs + TT * dimP;        // [TT][dimP]
   float* vs = ds + TT * dimP;        // [TT][CPB]
   float* bs = vs + TT * CPB;         // [TT]
+  float* gs = bs + TT;               // [TT] one decay per token (DECAY 2)
   const int b = blockIdx.z, h = blockIdx.y, hq = h / a.qk_rep, tid = threadIdx.x;
   const int slot = a.state_slots[b];
   if (slot < 0) return;
@@ -311,12 +396,12 @@ __global__ __launch_bounds__(256) void stk_linear_scan_kernel(StkScanArgs a) {
   for (int j = 0; j < R; j++) S[j] = (!fresh && col && r * R + j < dim) ? sp[j] : 0.f;
   const float hd = a.head_decay ? a.head_decay[h] : 1.f;
   // rows of dim floats that start on 16 bytes are fetched four floats a load
-  const bool vec = dim % 4 == 0 && a.ldk % 4 == 0 && a.ldq % 4 == 0 && (!DECAY || a.ldd % 4 == 0) && ((uintptr_t)a.k % 16) == 0 && ((uintptr_t)a.q % 16) == 0 &&
-                   (!DECAY || ((uintptr_t)a.decay % 16) == 0);
+  const bool vec = dim % 4 == 0 && a.ldk % 4 == 0 && a.ldq % 4 == 0 && (DECAY != 1 || a.ldd % 4 == 0) && ((uintptr_t)a.k % 16) == 0 && ((uintptr_t)a.q % 16) == 0 &&
+                   (DECAY != 1 || ((uintptr_t)a.decay % 16) == 0);
   // A tile's q, k, decays, values and write strengths travel global memory -> registers -> LDS; the registers of the NEXT tile are requested
   // before the current tile's tokens run, so their way from memory lies beside the arithmetic.
   float4 kn[NL], qn[NL], dn[NL];
-  float vbuf[16], bn = 0.f;
+  float vbuf[16], bn = 0.f, gn = 1.f;
   constexpr int vcount = TT * CPB;     // values of a tile: a thread takes elements tid, tid + 256, ... (at most 16)
   auto row4 = [&](const float* base, int ld, int hh, size_t t, int d, float fill) {
     const float* p = base + t * ld + hh * dim + d;
@@ -335,7 +420,7 @@ __global__ __launch_bounds__(256) void stk_linear_scan_kernel(StkScanArgs a) {
         const size_t t = (size_t)(t0 + i0 + i);
         kn[u] = row4(a.k, a.ldk, hq, t, d, 0.f);
         qn[u] = row4(a.q, a.ldq, hq, t, d, 0.f);
-        if (DECAY) dn[u] = row4(a.decay, a.ldd, h, t, d, 1.f);
+        if (DECAY == 1) dn[u] = row4(a.decay, a.ldd, h, t, d, 1.f);
       }
     }
 #pragma unroll
@@ -347,25 +432,31 @@ __global__ __launch_bounds__(256) void stk_linear_scan_kernel(StkScanArgs a) {
       }
     }
     if (BETA && tid < nt) bn = a.beta[(size_t)(t0 + i0 + tid) * a.ldb + h];
+    if (DECAY == 2 && tid < nt) gn = a.decay[(size_t)(t0 + i0 + tid) * a.ldd + h];
   };
   auto deposit = [&]() {
 #pragma unroll
     for (int u = 0; u < NL; u++) {
       const int e = tid + u * 256;
       if (e < TT * d4n) {
-        *(float4*)(ks + e * 4) = kn[u];
-        float4 qv = qn[u];
+        float4 kk = kn[u], qv = qn[u];
+        if (ACT) {
+          kk.x = siluf_(kk.x), kk.y = siluf_(kk.y), kk.z = siluf_(kk.z), kk.w = siluf_(kk.w);
+          qv.x = siluf_(qv.x), qv.y = siluf_(qv.y), qv.z = siluf_(qv.z), qv.w = siluf_(qv.w);
+        }
+        *(float4*)(ks + e * 4) = kk;
         qv.x *= a.q_scale, qv.y *= a.q_scale, qv.z *= a.q_scale, qv.w *= a.q_scale;
         *(float4*)(qs + e * 4) = qv;
-        if (DECAY) *(float4*)(ds + e * 4) = dn[u];
+        if (DECAY == 1) *(float4*)(ds + e * 4) = dn[u];
       }
     }
 #pragma unroll
     for (int u = 0; u < 16; u++) {
       const int e = tid + u * 256;
-      if (e < vcount) vs[e] = vbuf[u];
+      if (e < vcount) vs[e] = ACT ? siluf_(vbuf[u]) : vbuf[u];
     }
     if (BETA && tid < TT) bs[tid] = bn;
+    if (DECAY == 2 && tid < TT) gs[tid] = gn;
   };
   request(0);
   for (int i0 = 0; i0 < n; i0 += TT) {
@@ -375,24 +466,25 @@ __global__ __launch_bounds__(256) void stk_linear_scan_kernel(StkScanArgs a) {
     __syncthreads();
     if (i0 + TT < n) request(i0 + TT);
     // a token's operands come from LDS one token ahead of its arithmetic (two register sets, 16-byte reads)
-    float kv[2][R], qv[2][R], dv[2][R], uv[2], bv[2];
+    float kv[2][R], qv[2][R], dv[2][R], uv[2], bv[2], gv[2];
     auto fetch = [&](int i, int w) {
 #pragma unroll
       for (int j = 0; j < R; j += 4) {
         const float4 k4 = *(const float4*)(ks + i * dimP + r * R + j), q4 = *(const float4*)(qs + i * dimP + r * R + j);
         kv[w][j] = k4.x, kv[w][j + 1] = k4.y, kv[w][j + 2] = k4.z, kv[w][j + 3] = k4.w;
         qv[w][j] = q4.x, qv[w][j + 1] = q4.y, qv[w][j + 2] = q4.z, qv[w][j + 3] = q4.w;
-        if (DECAY) {
+        if (DECAY == 1) {
           const float4 d4 = *(const float4*)(ds + i * dimP + r * R + j);
           dv[w][j] = d4.x, dv[w][j + 1] = d4.y, dv[w][j + 2] = d4.z, dv[w][j + 3] = d4.w;
         }
       }
       uv[w] = vs[i * CPB + cl];
       if (BETA) bv[w] = bs[i];
+      if (DECAY == 2) gv[w] = gs[i];
     };
     auto token = [&](int i, int w) {
 #pragma unroll
-      for (int j = 0; j < R; j++) S[j] *= DECAY ? dv[w][j] : hd;
+      for (int j = 0; j < R; j++) S[j] *= DECAY == 1 ? dv[w][j] : (DECAY == 2 ? gv[w] : hd);
       float u = uv[w];
       if (BETA) {
         float d0 = 0.f, d1 = 0.f;  // (two chains; their sum order is fixed)
@@ -434,6 +526,23 @@ template <typename T>
 __global__ __launch_bounds__(256) void stk_head_norm_gate_kernel(const float* o, const float* w, const float* gate, int gate_ld, int gate_act, float eps,
                                                                  T* out, int H, int vdim) {
   const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (H == 1) {  // one norm over the whole row: the four waves share it
+    __shared__ float red[4];
+    const float* src = o + (size_t)t * vdim;
+    float s = 0.f;
+    for (int c = threadIdx.x; c < vdim; c += 256) s = fmaf(src[c], src[c], s);
+    const float r = 1.f / sqrtf(block_sum_256(s, red) / (float)vdim + eps);
+    for (int c = threadIdx.x; c < vdim; c += 256) {
+      float v = src[c] * r;
+      if (w) v *= w[c];
+      if (gate) {
+        const float g = gate[(size_t)t * gate_ld + c];
+        v *= gate_act == 1 ? siluf_(g) : sigmoidf_(g);
+      }
+      El<T>::st(out + (size_t)t * vdim + c, v);
+    }
+    return;
+  }
   for (int h = wave; h < H; h += 4) {
     const float* src = o + ((size_t)t * H + h) * vdim;
     float s = 0.f;
@@ -451,6 +560,95 @@ __global__ __launch_bounds__(256) void stk_head_norm_gate_kernel(const float* o,
   }
 }
 
+// ------------------------------------------------------------------------------------------------ short causal convolution with its state
+__global__ __launch_bounds__(256) void stk_conv_rows_kernel(StkConvArgs a) {
+  const int t = blockIdx.x, C = a.C, taps = a.taps;
+  const int b = seq_of_row(a.cu_q, a.B, t);
+  const int slot = a.state_slots[b];
+  if (slot < 0) return;
+  const int t0 = a.cu_q ? (int)a.cu_q[b] : t;
+  const int i = t - t0;
+  const bool fresh = a.positions[t0] == 0;
+  const float* cs = a.conv_state + (size_t)slot * (taps - 1) * C;
+  for (int c = blockIdx.y * 256 + threadIdx.x; c < C; c += 256 * gridDim.y) {
+    float y = a.bias ? a.bias[c] : 0.f;
+    for (int j = 0; j < taps; j++) {
+      const int e = i - (taps - 1) + j;
+      const bool from_step = e >= 0, counts = from_step || (!fresh && taps > 1);
+      const float* src = from_step ? a.x + (size_t)(t0 + e) * a.ld : (counts ? cs + (size_t)(taps - 1 + e) * C : a.x + (size_t)t * a.ld);
+      const float wv = counts ? a.w[(size_t)c * taps + j] : 0.f;
+      y = fmaf(wv, src[c], y);
+    }
+    a.y[(size_t)t * a.ldy + c] = a.act == 1 ? siluf_(y) : y;
+  }
+}
+__global__ __launch_bounds__(256) void stk_conv_rows_update_kernel(StkConvArgs a) {
+  const int b = blockIdx.x;
+  const int slot = a.state_slots[b];
+  if (slot < 0) return;
+  const int C = a.C, taps = a.taps;
+  const int t0 = a.cu_q ? (int)a.cu_q[b] : b, n = a.cu_q ? (int)a.cu_q[b + 1] - t0 : 1;
+  const bool fresh = a.positions[t0] == 0;
+  float* cs = a.conv_state + (size_t)slot * (taps - 1) * C;
+  for (int c = blockIdx.y * 256 + threadIdx.x; c < C; c += 256 * gridDim.y)
+    for (int r = 0; r < taps - 1; r++) {  // (rows are read above where they are written)
+      const int e = n - (taps - 1) + r;
+      float v = 0.f;
+      if (e >= 0) v = a.x[(size_t)(t0 + e) * a.ld + c];
+      else if (!fresh) v = cs[(size_t)(taps - 1 + e) * C + c];
+      cs[(size_t)r * C + c] = v;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ real-gated diagonal recurrence
+// lane = channel, a sequence's tokens in order.  The operands of GT tokens are requested together and a tile ahead; gates, decay and input
+// weight of a tile are formed before its GT dependent multiply-adds run, so only those wait for one another.
+__device__ __forceinline__ float gelu_tanhf_(float z) {
+  return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+template <typename T>
+__global__ __launch_bounds__(64) void stk_gated_scan_kernel(StkGatedScanArgs a) {
+  constexpr int GT = 8;
+  const int b = blockIdx.y, c = blockIdx.x * 64 + threadIdx.x;
+  const int slot = a.state_slots[b];
+  if (slot < 0 || c >= a.C) return;
+  const int t0 = a.cu_q ? (int)a.cu_q[b] : b, n = a.cu_q ? (int)a.cu_q[b + 1] - t0 : 1;
+  const bool fresh = a.positions[t0] == 0;
+  float* sp = a.state + (size_t)slot * a.C + c;
+  float S = fresh ? 0.f : *sp;
+  const float sl = a.rate * softplusf_(a.lam[c]);
+  const int gc = a.block > 0 ? c / a.block * 2 * a.block + c % a.block : c;
+  T* out = (T*)a.out;
+  float un[GT], rn[GT], in_[GT], yn[GT];
+  auto request = [&](int i0) {
+#pragma unroll
+    for (int j = 0; j < GT; j++) {
+      const size_t t = (size_t)(t0 + min(i0 + j, n - 1));
+      un[j] = a.u[t * a.ldu + c], rn[j] = a.gr[t * a.ldg + gc], in_[j] = a.gi[t * a.ldg + gc], yn[j] = a.y[t * a.ldy + c];
+    }
+  };
+  request(0);
+  for (int i0 = 0; i0 < n; i0 += GT) {
+    float av[GT], bv[GT], yv[GT];
+#pragma unroll
+    for (int j = 0; j < GT; j++) {
+      const float la = -sl * sigmoidf_(rn[j]), aj = expf(la);
+      av[j] = aj;
+      bv[j] = sqrtf(-expm1f(2.f * la)) * (sigmoidf_(in_[j]) * un[j]);  // (1 - a^2 without the cancellation near a = 1)
+      yv[j] = gelu_tanhf_(yn[j]);
+    }
+    if (i0 + GT < n) request(i0 + GT);
+#pragma unroll
+    for (int j = 0; j < GT; j++) {
+      if (i0 + j < n) {
+        S = fmaf(av[j], S, bv[j]);
+        El<T>::st(out + (size_t)(t0 + i0 + j) * a.ldo + c, S * yv[j]);
+      }
+    }
+  }
+  *sp = S;
+}
+
 }  // namespace
 
 // ================================================================================================ launchers
@@ -466,7 +664,13 @@ void vra_stack_embed_pair(const StkEmbedPairArgs& a, int dtype, int64_t stream) 
 void vra_stack_sandwich_norm(const StkSandwichArgs& a, int dtype, int64_t stream) {
   VRA_CHECK_ARG(a.x && a.T > 0 && a.W > 0 && (!a.post_w || (a.p1 && a.n1 >= 1)) && (!a.pre_w || a.h), "stack seam norm: null pointer or empty shape");
   VRA_CHECK_ARG(!a.router_w || (a.pre_w && a.pair_expert && a.pair_weight && a.top >= 1 && a.top <= a.n_router), "stack seam norm: router outputs");
-  const size_t lds = ((size_t)a.W + a.n_router + 1) * sizeof(float);
+  VRA_CHECK_ARG(!a.dyt || ((!a.post_w || a.post_b) && (!a.pre_w || a.pre_b)), "stack seam norm: Dynamic Tanh needs its offsets");
+  VRA_CHECK_ARG((!a.p1_norm_w && !a.p2_norm_w) || a.n1 == 1, "stack seam norm: a part with a norm of its own is one row a token");
+  VRA_CHECK_ARG(a.router_kind == 0 || !a.router_w ||
+                    (a.n_identity >= 0 && a.n_identity < a.n_router && (a.n_groups <= 1 || (a.n_router % a.n_groups == 0 && a.keep >= 1)) &&
+                     (a.n_identity == 0 || a.id_weight)),
+                "stack seam norm: router groups / identity experts");
+  const size_t lds = ((size_t)a.W + 2 * (size_t)a.n_router + (size_t)std::max(a.n_groups, 0) + 1) * sizeof(float);
   VRA_CHECK_ARG(lds <= 64 * 1024, "stack seam norm: row does not fit LDS");
   if (dtype == VRA_F32) launch_checked("stack seam norm", [&] { stk_sandwich_kernel<float><<<a.T, 256, lds, as_stream(stream)>>>(a); });
   else launch_checked("stack seam norm", [&] { stk_sandwich_kernel<uint16_t><<<a.T, 256, lds, as_stream(stream)>>>(a); });
@@ -510,16 +714,20 @@ void vra_stack_linear_scan(const StkScanArgs& a, int64_t stream) {
   int P = 1;
   while (P * R < a.dim) P <<= 1;
   const int CPB = 256 / P, dimP = P * R;
-  const size_t lds = ((size_t)16 * dimP * 3 + (size_t)16 * CPB + 16) * sizeof(float);
+  const size_t lds = ((size_t)16 * dimP * 3 + (size_t)16 * CPB + 32) * sizeof(float);
   dim3 grid((a.vdim + CPB - 1) / CPB, a.H, a.B);
   hipStream_t st = as_stream(stream);
-  const bool decay = a.decay != nullptr, beta = a.beta != nullptr;
+  const bool decay = a.decay != nullptr, beta = a.beta != nullptr, per_head = decay && a.decay_per_head;
   VRA_CHECK_ARG(decay || !beta, "stack linear scan: the delta rule comes with per-row decays");
+  VRA_CHECK_ARG(!a.act_silu || (!decay && !beta), "stack linear scan: the activation on the way in goes with constant decays");
+  VRA_CHECK_ARG(!per_head || beta, "stack linear scan: one decay per head and token goes with the delta rule");
 #define STK_SCAN(PV)                                                                                                            \
   launch_checked("stack linear scan", [&] {                                                                                     \
-    if (beta) stk_linear_scan_kernel<R, PV, true, true><<<grid, 256, lds, st>>>(a);                                             \
-    else if (decay) stk_linear_scan_kernel<R, PV, true, false><<<grid, 256, lds, st>>>(a);                                      \
-    else stk_linear_scan_kernel<R, PV, false, false><<<grid, 256, lds, st>>>(a);                                                \
+    if (per_head) stk_linear_scan_kernel<R, PV, 2, true, false><<<grid, 256, lds, st>>>(a);                                     \
+    else if (beta) stk_linear_scan_kernel<R, PV, 1, true, false><<<grid, 256, lds, st>>>(a);                                    \
+    else if (decay) stk_linear_scan_kernel<R, PV, 1, false, false><<<grid, 256, lds, st>>>(a);                                  \
+    else if (a.act_silu) stk_linear_scan_kernel<R, PV, 0, false, true><<<grid, 256, lds, st>>>(a);                              \
+    else stk_linear_scan_kernel<R, PV, 0, false, false><<<grid, 256, lds, st>>>(a);                                             \
   })
   switch (P) {
     case 1: STK_SCAN(1); break;
@@ -541,6 +749,29 @@ void vra_stack_head_norm_gate(const float* o, const float* w, const float* gate,
     launch_checked("stack head norm", [&] {
       stk_head_norm_gate_kernel<uint16_t><<<T, 256, 0, as_stream(stream)>>>(o, w, gate, gate_ld, gate_act, eps, (uint16_t*)out, H, vdim);
     });
+}
+
+void vra_stack_conv_rows(const StkConvArgs& a, int64_t stream) {
+  VRA_CHECK_ARG(a.x && a.w && a.y && a.positions && a.state_slots && (a.taps < 2 || a.conv_state), "stack convolution: null pointer");
+  VRA_CHECK_ARG(a.T > 0 && a.B > 0 && a.C > 0 && a.taps >= 1 && a.ld >= a.C && a.ldy >= a.C, "stack convolution: shapes");
+  StkConvArgs k = a;
+  if (!k.conv_state) k.conv_state = k.y;  // (one tap: never read)
+  const dim3 grid(a.T, std::min((a.C + 255) / 256, 64));
+  launch_checked("stack convolution", [&] { stk_conv_rows_kernel<<<grid, 256, 0, as_stream(stream)>>>(k); });
+}
+void vra_stack_conv_rows_update(const StkConvArgs& a, int64_t stream) {
+  VRA_CHECK_ARG(a.x && a.positions && a.state_slots && a.B > 0 && a.taps >= 1 && a.C > 0, "stack convolution state: null pointer or empty shape");
+  if (a.taps < 2) return;
+  VRA_CHECK_ARG(a.conv_state, "stack convolution state: null pointer");
+  const dim3 grid(a.B, std::min((a.C + 255) / 256, 64));
+  launch_checked("stack convolution state", [&] { stk_conv_rows_update_kernel<<<grid, 256, 0, as_stream(stream)>>>(a); });
+}
+void vra_stack_gated_scan(const StkGatedScanArgs& a, int dtype, int64_t stream) {
+  VRA_CHECK_ARG(a.u && a.gr && a.gi && a.y && a.lam && a.state && a.state_slots && a.positions && a.out, "stack gated scan: null pointer");
+  VRA_CHECK_ARG(a.B > 0 && a.C > 0 && a.ldu >= a.C && a.ldy >= a.C && a.ldo >= a.C, "stack gated scan: shapes");
+  const dim3 grid((a.C + 63) / 64, a.B);
+  if (dtype == VRA_F32) launch_checked("stack gated scan", [&] { stk_gated_scan_kernel<float><<<grid, 64, 0, as_stream(stream)>>>(a); });
+  else launch_checked("stack gated scan", [&] { stk_gated_scan_kernel<uint16_t><<<grid, 64, 0, as_stream(stream)>>>(a); });
 }
 
 // ================================================================================================ C entry points (operator tests)

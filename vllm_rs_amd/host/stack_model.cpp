@@ -70,13 +70,14 @@ bool StackModel::parse_spec(const char* spec) {
         return false;
       norm_offset_ = (float)num("norm_offset", 0.0), embed_scale_ = (float)num("embed_scale", 1.0), embed_norm_ = (int)num("embed_norm", 0);
       pair_buckets_ = (int)num("pair_buckets", 0), pair_mul_prev_ = (int64_t)num("pair_mul_prev", 0), pair_mul_cur_ = (int64_t)num("pair_mul_cur", 0);
+      tie_head_ = (int)num("tie_head", 0);
     } else if (kind == "layer") {
       StackLayer L;
       L.heads = (int)num("heads", 0), L.kv_heads = (int)num("kv_heads", L.heads), L.dim = (int)num("dim", 0), L.vdim = (int)num("vdim", L.dim);
       L.scale = (float)num("scale", L.dim > 0 ? 1.0 / sqrt((double)L.dim) : 1.0), L.softcap = (float)num("softcap", 0.0);
       L.temp_coef = (float)num("temp_coef", 0.0), L.temp_every = (int)num("temp_every", 0), L.kv_from = (int)num("kv_from", -1);
       const std::string mix = f.count("mixer") ? f["mixer"] : "attention";
-      L.mixer = mix == "latent" ? 1 : (mix == "sigmoid" ? 2 : (mix == "delta" ? 3 : (mix == "retention" ? 4 : (mix == "parallel" ? 5 : 0))));
+      L.mixer = mix == "latent" ? 1 : (mix == "sigmoid" ? 2 : (mix == "delta" ? 3 : (mix == "retention" ? 4 : (mix == "parallel" ? 5 : (mix == "lightning" ? 6 : 0)))));
       if (mix != "attention" && L.mixer == 0) return spec_error_ = "layer stack spec: unknown mixer " + mix, false;
       L.conv = (int)num("conv", 0), L.rank_a = (int)num("rank_a", 0), L.rank_g = (int)num("rank_g", 0), L.chunk = (int)num("chunk", 0);
       L.qk_norm = (int)num("qk_norm", 0), L.has_bias = (int)num("bias", 0);
@@ -90,8 +91,18 @@ bool StackModel::parse_spec(const char* spec) {
       }
       {
         const std::string rk = f.count("router") ? f["router"] : "sigmoid", ak = f.count("act") ? f["act"] : "clamped";
-        if ((rk != "sigmoid" && rk != "softmax") || (ak != "clamped" && ak != "silu")) return spec_error_ = "layer stack spec: router is sigmoid or softmax, act clamped or silu", false;
-        L.router_kind = rk == "softmax", L.act_kind = ak == "silu" ? 2 : 0;
+        if ((rk != "sigmoid" && rk != "softmax" && rk != "softmax_all") || (ak != "clamped" && ak != "silu"))
+          return spec_error_ = "layer stack spec: router is sigmoid, softmax or softmax_all, act clamped or silu", false;
+        L.router_kind = rk == "softmax" ? 1 : (rk == "softmax_all" ? 2 : 0), L.act_kind = ak == "silu" ? 2 : 0;
+        L.n_identity = (int)num("identity", 0), L.n_groups = (int)num("groups", 0), L.keep = (int)num("keep", 0);
+      }
+      {
+        const std::string rt = f.count("right") ? f["right"] : "gla", rl = f.count("rot_layout") ? f["rot_layout"] : "half";
+        if ((rt != "gla" && rt != "rglru") || (rl != "half" && rl != "pairs")) return spec_error_ = "layer stack spec: right is gla or rglru, rot_layout half or pairs", false;
+        L.right_kind = rt == "rglru", L.rot_layout = rl == "pairs";
+        L.lowrank = (int)num("lowrank", 1), L.r_width = (int)num("r_width", 0), L.r_blocks = (int)num("r_blocks", 1);
+        L.head_temp = (int)num("head_temp", 0), L.head_gate = (int)num("head_gate", 0), L.branch_norm = (int)num("branch_norm", 0);
+        if (L.right_kind == 1) L.conv = (int)num("r_conv", 1);
       }
       L.weights_of = (int)num("weights_of", -1);
       L.rot_dim = (int)num("rot_dim", 0), L.kv_rank = (int)num("kv_rank", 0), L.q_rank = (int)num("q_rank", 0), L.rot_dims = (int)num("rot_dims", L.rot_dim);
@@ -99,8 +110,8 @@ bool StackModel::parse_spec(const char* spec) {
       L.yarn_original = num("yarn_original", 0.0), L.yarn_fast = num("yarn_fast", 32.0), L.yarn_slow = num("yarn_slow", 1.0);
       L.window = (int)num("window", 0), L.keep_first = (int)num("keep_first", 0), L.slope_exp = num("slope_exp", 0.0);
       const std::string mlp = f.count("mlp") ? f["mlp"] : "none";
-      L.mlp = mlp == "dense" ? 1 : (mlp == "moe" ? 2 : (mlp == "gated" ? 3 : 0));
-      if (mlp != "dense" && mlp != "moe" && mlp != "none" && mlp != "gated") return spec_error_ = "layer stack spec: unknown feed-forward kind " + mlp, false;
+      L.mlp = mlp == "dense" ? 1 : (mlp == "moe" ? 2 : (mlp == "gated" ? 3 : (mlp == "clamped" ? 4 : 0)));
+      if (mlp != "dense" && mlp != "moe" && mlp != "none" && mlp != "gated" && mlp != "clamped") return spec_error_ = "layer stack spec: unknown feed-forward kind " + mlp, false;
       L.ff = (int)num("ff", 0), L.experts = (int)num("experts", 0), L.top = (int)num("top", 1), L.limit = (float)num("limit", 0.0);
       L.shared_ff = (int)num("shared_ff", 0), L.shared_limit = (float)num("shared_limit", 0.0);
       layers_.push_back(L);
@@ -120,15 +131,27 @@ bool StackModel::parse_spec(const char* spec) {
     if ((L.mixer == 1 || L.mixer == 2) && block_ != 1) return spec_error_ = "layer stack spec: latent and sigmoid mixers run in sequential blocks" + at, false;
     if (L.mixer == 0 && block_ != 0) return spec_error_ = "layer stack spec: the softmax mixer with temperature and cap runs in parallel blocks" + at, false;
     if (L.mixer >= 3 && block_ != 2) return spec_error_ = "layer stack spec: delta, retention and parallel mixers run in sandwich blocks" + at, false;
-    if (block_ == 2 && (L.mixer < 3 || (L.mlp != 0 && L.mlp != 2) || L.weights_of >= 0))
-      return spec_error_ = "layer stack spec: sandwich blocks hold delta, retention or parallel mixers and a mixture of experts or no feed-forward" + at, false;
-    if (L.mixer == 3 && (L.conv < 1 || L.rank_a < 1 || L.rank_g < 1 || L.dim > 256)) return spec_error_ = "layer stack spec: the delta mixer needs conv >= 1, rank_a, rank_g, dim <= 256" + at, false;
+    if (block_ == 2 && (L.mixer < 3 || (L.mlp != 0 && L.mlp != 2 && L.mlp != 4) || L.weights_of >= 0))
+      return spec_error_ = "layer stack spec: sandwich blocks hold delta, retention, lightning or parallel mixers and a mixture of experts, a clamped dense feed-forward or none" + at, false;
+    if (L.mlp == 4 && block_ != 2) return spec_error_ = "layer stack spec: the clamped dense feed-forward belongs to sandwich blocks" + at, false;
+    if (L.mixer == 3 && (L.conv < 1 || (L.lowrank && (L.rank_a < 1 || L.rank_g < 1)) || L.dim > 256)) return spec_error_ = "layer stack spec: the delta mixer needs conv >= 1, rank_a, rank_g, dim <= 256" + at, false;
+    if (L.mixer == 6 && ((int)L.decay.size() != L.heads || L.kv_heads != L.heads || L.dim > 256))
+      return spec_error_ = "layer stack spec: lightning needs one decay per head, kv_heads = heads, dim <= 256" + at, false;
+    if (L.mixer == 5 && L.right_kind == 1 &&
+        (L.r_width <= 0 || L.r_blocks < 1 || L.r_width % L.r_blocks || L.conv < 1 || L.rot_dims < 0 || L.rot_dims > L.dim || L.rot_dims % 2 || L.chunk < 0 ||
+         L.window < 0 || L.vdim > 256 || (L.yarn_factor > 0.0 && (L.yarn_original <= 0.0 || L.yarn_fast <= 0.0 || L.yarn_slow <= 0.0))))
+      return spec_error_ = "layer stack spec: the parallel mixer with a gated recurrence needs r_width in r_blocks equal blocks, r_conv >= 1, an even rot_dims <= dim, vdim <= 256" + at, false;
+    if ((L.window > 0 || L.head_temp || L.head_gate || L.rot_layout || L.branch_norm) && L.mixer != 5 && L.mixer != 2)
+      return spec_error_ = "layer stack spec: window, head_temp, head_gate, rot_layout and branch_norm belong to the parallel mixer" + at, false;
+    if (L.router_kind == 2 && (L.n_identity < 0 ||
+                               (L.n_groups > 1 && ((L.experts + L.n_identity) % L.n_groups || L.keep < 1 || L.keep > L.n_groups))))
+      return spec_error_ = "layer stack spec: router groups must divide experts + identity, 1 <= keep <= groups" + at, false;
     if (L.mixer == 4 && ((int)L.decay.size() != L.heads || L.kv_heads != L.heads || L.rot_dims < 0 || L.rot_dims > L.dim || L.rot_dims % 2 || L.dim > 256))
       return spec_error_ = "layer stack spec: retention needs one decay per head, kv_heads = heads, an even rot_dims <= dim <= 256" + at, false;
-    if (L.mixer == 5 && (L.r_heads <= 0 || L.r_dim <= 0 || L.r_dim > 256 || L.r_vdim <= 0 || L.rank_a < 1 || !(L.tau > 0.f) || L.rot_dims < 0 || L.rot_dims > L.dim || L.rot_dims % 2 ||
+    if (L.mixer == 5 && L.right_kind == 0 && (L.r_heads <= 0 || L.r_dim <= 0 || L.r_dim > 256 || L.r_vdim <= 0 || L.rank_a < 1 || !(L.tau > 0.f) || L.rot_dims < 0 || L.rot_dims > L.dim || L.rot_dims % 2 ||
                          L.chunk < 0 || L.vdim > 256 || (L.rs_factor > 0.0 && (L.rs_original <= 0.0 || L.rs_high <= L.rs_low))))
       return spec_error_ = "layer stack spec: the parallel mixer needs r_heads, r_dim <= 256, r_vdim, rank_a, tau > 0, an even rot_dims <= dim, vdim <= 256" + at, false;
-    if (L.router_kind == 1 && (block_ != 2 || L.shared_ff > 0)) return spec_error_ = "layer stack spec: the softmax router belongs to sandwich blocks and has no shared expert" + at, false;
+    if (L.router_kind >= 1 && (block_ != 2 || L.shared_ff > 0)) return spec_error_ = "layer stack spec: the softmax router belongs to sandwich blocks and has no shared expert" + at, false;
     if (L.mixer != 0 && L.kv_from >= 0) return spec_error_ = "layer stack spec: kv_from belongs to the softmax mixer" + at, false;
     if (L.mixer == 1 && (L.kv_rank <= 0 || L.q_rank <= 0 || L.rot_dim < 0 || L.kv_rank > 256 || L.rot_dims < 0 || L.rot_dims > L.rot_dim || L.rot_dims % 2 ||
                          (L.yarn_factor > 0.0 && (L.yarn_original <= 0.0 || L.yarn_fast <= 0.0 || L.yarn_slow <= 0.0))))
@@ -160,9 +183,10 @@ bool StackModel::parse_spec(const char* spec) {
     }
     if (!L.has_cache()) L.owns_cache = false;  // (their past lives in the state slot; the cache entry keeps the tables uniform and holds no bytes)
     if (L.mlp == 1 && L.ff <= 0) return spec_error_ = "layer stack spec: dense feed-forward without ff" + at, false;
-    if (L.mlp == 2 && (L.ff <= 0 || L.experts <= 0 || L.top < 1 || L.top > L.experts))
+    if (L.mlp == 2 && (L.ff <= 0 || L.experts <= 0 || L.top < 1 || L.top > L.experts + L.n_identity))
       return spec_error_ = "layer stack spec: mixture of experts needs ff, experts and 1 <= top <= experts" + at, false;
-    if (L.mlp == 3) {
+    if (L.mlp == 4 && L.ff <= 0) return spec_error_ = "layer stack spec: clamped feed-forward without ff" + at, false;
+    if (L.mlp == 3 || L.mlp == 4) {
       if (L.ff <= 0) return spec_error_ = "layer stack spec: gated feed-forward without ff" + at, false;
       L.shared_ff = L.ff;  // (laid out like a shared expert: gate / up rows interleaved, one weight set for all rows)
     }
@@ -320,8 +344,12 @@ bool StackModel::finalize_weights() {
     if (it == staged_.end() || it->second.shape.size() != 2 || it->second.shape[1] != cols) return -1;
     return it->second.shape[0];
   };
-  if (!up_mat("embed", vocab_, W, &embed_) || !up_mat("head", vocab_, W, &head_)) return false;
-  if (block_ == 2) {
+  if (!up_mat("embed", vocab_, W, &embed_)) return false;
+  if (tie_head_) head_ = embed_;
+  else if (!up_mat("head", vocab_, W, &head_)) return false;
+  if (block_ == 2 && norm_kind_ == 1) {
+    if (!up_norm("final.norm", &final_norm_, &final_b_, &final_alpha_)) return false;
+  } else if (block_ == 2) {
     if (!up_norm_off("final.norm", W, &final_norm_)) return false;
     if (embed_norm_ && !up_norm_off("embed.norm", W, &embed_norm_w_)) return false;
     if (pair_buckets_ > 0 && !up_mat("bigram", (int64_t)pair_buckets_ + 1, W, &pair_table_)) return false;
@@ -332,7 +360,10 @@ bool StackModel::finalize_weights() {
     StackLayer& L = layers_[li];
     if (L.weights_of >= 0) continue;
     const std::string p = "l" + std::to_string(li) + ".";
-    if (block_ == 2) {
+    if (block_ == 2 && norm_kind_ == 1) {
+      if (!up_norm(p + "norm1", &L.norm_w, &L.norm_b, &L.norm_alpha) || !up_norm(p + "norm1b", &L.post1_w, &L.post1_b, &L.post1_alpha)) return false;
+      if (L.mlp != 0 && (!up_norm(p + "norm2", &L.norm2_w, &L.norm2_b, &L.norm2_alpha) || !up_norm(p + "norm2b", &L.post2_w, &L.post2_b, &L.post2_alpha))) return false;
+    } else if (block_ == 2) {
       if (!up_norm_off(p + "norm1", W, &L.norm_w) || !up_norm_off(p + "norm1b", W, &L.post1_w)) return false;
       if (L.mlp != 0 && (!up_norm_off(p + "norm2", W, &L.norm2_w) || !up_norm_off(p + "norm2b", W, &L.post2_w))) return false;
     } else {
@@ -348,7 +379,86 @@ bool StackModel::finalize_weights() {
       weight_bytes_ += m.size();
       return (*dst = upload(m.data(), m.size())) != nullptr;
     };
-    if (L.mixer == 3) {
+    auto conv_taps = [&](const std::string& name) {  // the taps of a short convolution are the columns of its tensor
+      auto it = staged_.find(name);
+      if (it != staged_.end() && it->second.shape.size() == 2 && it->second.shape[1] >= 1) L.conv = (int)it->second.shape[1];
+    };
+    if (L.mixer == 3 && !L.lowrank) {
+      // gated delta rule with full-rank side projections: q | k | v | write strengths | decays | gate in one matrix
+      const int H = L.heads, nk = L.nk(), nv = H * L.vdim, C = L.conv_channels();
+      conv_taps(p + "mix.q.conv");
+      const HostTensor *q, *k, *v, *bw, *aw, *gw, *cq, *ck, *cv, *al;
+      if (!need(p + "mix.q", nk, W, &q) || !need(p + "mix.k", nk, W, &k) || !need(p + "mix.v", nv, W, &v) || !need(p + "mix.b", H, W, &bw) ||
+          !need(p + "mix.a", H, W, &aw) || !need(p + "mix.g", nv, W, &gw) || !matrix(q) || !matrix(k) || !matrix(v) || !matrix(bw) || !matrix(aw) || !matrix(gw))
+        return false;
+      if (!up_rows({q, k, v, bw, aw, gw}, &L.qkv)) return false;
+      if (!need(p + "mix.q.conv", nk, L.conv, &cq) || !need(p + "mix.k.conv", nk, L.conv, &ck) || !need(p + "mix.v.conv", nv, L.conv, &cv)) return false;
+      std::vector<float> cw;
+      f32_of(*cq, &cw), f32_of(*ck, &cw), f32_of(*cv, &cw);
+      if ((int)cw.size() != C * L.conv || !(L.conv_w = upload_floats(cw))) return false;
+      if (!need(p + "mix.A_log", H, -1, &al)) return false;
+      std::vector<float> rate;
+      f32_of(*al, &rate);
+      for (float& r : rate) r = expf(r);
+      if (!(L.rate = upload_floats(rate)) || !up_vec(p + "mix.dt_bias", H, &L.dt_bias) || !up_vec(p + "mix.norm", L.vdim, &L.out_norm_w)) return false;
+      if (!up_mat(p + "mix.o", W, nv, &L.o)) return false;
+    } else if (L.mixer == 6) {
+      const int H = L.heads;
+      const HostTensor *q, *k, *v, *g;
+      if (!need(p + "mix.q", (int64_t)H * L.dim, W, &q) || !need(p + "mix.k", (int64_t)H * L.dim, W, &k) || !need(p + "mix.v", (int64_t)H * L.vdim, W, &v) ||
+          !need(p + "mix.g", (int64_t)H * L.vdim, W, &g) || !matrix(q) || !matrix(k) || !matrix(v) || !matrix(g))
+        return false;
+      if (!up_rows({q, k, v, g}, &L.qkv) || !(L.head_decay = upload_floats(L.decay)) || !up_mat(p + "mix.o", W, H * L.vdim, &L.o) ||
+          !up_vec(p + "mix.norm", (int64_t)H * L.vdim, &L.out_norm_w))
+        return false;
+    } else if (L.mixer == 5 && L.right_kind == 1) {
+      const std::string pl = p + "mix.left.", pr = p + "mix.right.";
+      const int H = L.heads, Wr = L.r_width, nb = L.r_blocks, bw = Wr / nb;
+      conv_taps(pr + "conv");
+      const HostTensor *q, *k, *v, *g = nullptr, *y, *xr, *cw, *ra, *ri, *rab, *rib;
+      if (!need(pl + "q", L.nq(), W, &q) || !need(pl + "k", L.nk(), W, &k) || !need(pl + "v", L.nv(), W, &v) || !need(pr + "y", Wr, W, &y) ||
+          !need(pr + "x", Wr, W, &xr) || !matrix(q) || !matrix(k) || !matrix(v) || !matrix(y) || !matrix(xr))
+        return false;
+      if (L.head_gate && (!need(pl + "g", H, W, &g) || !matrix(g))) return false;
+      std::vector<const HostTensor*> parts{q, k, v};
+      if (g) parts.push_back(g);
+      parts.push_back(y), parts.push_back(xr);
+      if (!up_rows(parts, &L.qkv)) return false;
+      std::vector<float> bias;
+      if (L.has_bias) {
+        const HostTensor *qb, *kb, *vb;
+        if (!need(pl + "q.b", L.nq(), -1, &qb) || !need(pl + "k.b", L.nk(), -1, &kb) || !need(pl + "v.b", L.nv(), -1, &vb)) return false;
+        f32_of(*qb, &bias), f32_of(*kb, &bias), f32_of(*vb, &bias);
+      }
+      bias.resize(L.nq() + L.nk() + L.nv() + (g ? H : 0), 0.f);
+      {
+        const HostTensor *yb, *xb;
+        if (!need(pr + "y.b", Wr, -1, &yb) || !need(pr + "x.b", Wr, -1, &xb)) return false;
+        f32_of(*yb, &bias), f32_of(*xb, &bias);
+      }
+      if ((int)bias.size() != L.nqkv() || !(L.qkv_bias = upload_floats(bias))) return false;
+      if (L.qk_norm && (!up_vec(pl + "q.norm", L.dim, &L.qn_w) || !up_vec(pl + "k.norm", L.dim, &L.kn_w))) return false;
+      if (L.head_temp && !up_vec(pl + "temp", H, &L.temp_w)) return false;
+      if (L.sink && !up_vec(pl + "sink", H, &L.sink_w)) return false;
+      if (L.branch_norm && (!up_vec(pl + "out", W, &L.left_out_w) || !up_vec(pr + "out", W, &L.right_out_w))) return false;
+      if (!up_mat(pl + "o", W, H * L.vdim, &L.o) || !up_mat(pr + "o", W, Wr, &L.r_o)) return false;
+      if (!need(pr + "conv", Wr, L.conv, &cw) || !(L.conv_w = upload_f32(*cw)) || !up_vec(pr + "conv.b", Wr, &L.conv_b) || !up_vec(pr + "lam", Wr, &L.lam)) return false;
+      // the gates of the recurrence are computed in f32: per block the rows of the recurrence gate, then those of the input gate
+      if (!need(pr + "ra", (int64_t)nb * bw * bw, -1, &ra) || !need(pr + "ri", (int64_t)nb * bw * bw, -1, &ri) || !need(pr + "ra.b", Wr, -1, &rab) ||
+          !need(pr + "ri.b", Wr, -1, &rib))
+        return false;
+      std::vector<float> fa, fi, ba, bi, gw, gb;
+      f32_of(*ra, &fa), f32_of(*ri, &fi), f32_of(*rab, &ba), f32_of(*rib, &bi);
+      for (int b = 0; b < nb; b++) {
+        gw.insert(gw.end(), fa.begin() + (size_t)b * bw * bw, fa.begin() + (size_t)(b + 1) * bw * bw);
+        gw.insert(gw.end(), fi.begin() + (size_t)b * bw * bw, fi.begin() + (size_t)(b + 1) * bw * bw);
+        gb.insert(gb.end(), ba.begin() + (size_t)b * bw, ba.begin() + (size_t)(b + 1) * bw);
+        gb.insert(gb.end(), bi.begin() + (size_t)b * bw, bi.begin() + (size_t)(b + 1) * bw);
+      }
+      if (!(L.gates_w = upload_floats(gw)) || !(L.gates_b = upload_floats(gb))) return false;
+      rotary_table(L);
+      if (!L.freq_hi || !L.freq_lo) return false;
+    } else if (L.mixer == 3) {
       // gated delta rule: q | k | v | write strengths in one matrix; the first stages of the decay and gate projections in a second one,
       // their second stages block-diagonal in a third
       const int H = L.heads, nk = L.nk(), nv = H * L.vdim, C = L.conv_channels();
@@ -479,7 +589,7 @@ bool StackModel::finalize_weights() {
     if (L.mixer < 3 && !up_mat(p + "mix.o", W, L.heads * L.vdim, &L.o)) return false;
     if (L.mlp == 1) {
       if (!up_mat(p + "mlp.up", L.ff, W, &L.up) || !up_mat(p + "mlp.down", W, L.ff, &L.down) || !up_vec(p + "mlp.act", 4, &L.act)) return false;
-    } else if (L.mlp == 3) {
+    } else if (L.mlp == 3 || L.mlp == 4) {
       const HostTensor *g, *u, *d;
       if (!need(p + "mlp.gate", L.ff, W, &g) || !need(p + "mlp.up", L.ff, W, &u) || !need(p + "mlp.down", W, L.ff, &d) || !matrix(g) || !matrix(u) || !matrix(d))
         return false;
@@ -490,13 +600,14 @@ bool StackModel::finalize_weights() {
       if (!(L.s_gu = upload(sgu.data(), sgu.size())) || !(L.s_down = upload(sdn.data(), sdn.size()))) return false;
     } else if (L.mlp == 2) {
       const HostTensor *r, *sg = nullptr;
-      if (!need(p + "mlp.router", L.experts, W, &r) || !matrix(r)) return false;
+      if (!need(p + "mlp.router", L.experts + L.n_identity, W, &r) || !matrix(r)) return false;
       if (L.shared_ff > 0 && (!need(p + "mlp.shared.sg", W, -1, &sg) || !matrix(sg))) return false;
       std::vector<uint8_t> rt(r->data);
       if (sg) rt.insert(rt.end(), sg->data.begin(), sg->data.end());
       weight_bytes_ += rt.size();
       if (!(L.router = upload(rt.data(), rt.size()))) return false;
       if (L.router_kind == 1 && !up_vec(p + "mlp.router.b", L.experts, &L.router_bias)) return false;
+      if (L.router_kind == 2 && !up_vec(p + "mlp.correction", L.experts + L.n_identity, &L.router_bias)) return false;
       std::vector<uint8_t> gu((size_t)L.experts * 2 * L.ffp * W * es), dn((size_t)L.experts * W * L.ffp * es);
       for (int e = 0; e < L.experts; e++) {
         const std::string pe = p + "mlp.e" + std::to_string(e) + ".";
@@ -567,12 +678,14 @@ bool StackModel::init_synthetic(uint64_t seed) {
   };
   const int W = width_;
   put("embed", vocab_, W, 0, 1.0);
-  put("head", vocab_, W, 0, 1.0 / sqrt((double)W));
+  if (!tie_head_) put("head", vocab_, W, 0, 1.0 / sqrt((double)W));
   auto put_norm = [&](const std::string& name) {
     put(name, W, 0, 1, 0.05);
     if (norm_kind_ == 1) put(name + ".b", W, 0, 0, 0.02), put(name + ".alpha", 1, 0, 0.5, 0.0);
   };
-  if (block_ == 2) {  // norm weights are stored around zero; the embedding's own norm and the token-pair table
+  if (block_ == 2 && norm_kind_ == 1) {
+    put_norm("final.norm");
+  } else if (block_ == 2) {  // norm weights are stored around zero; the embedding's own norm and the token-pair table
     put("final.norm", W, 0, 0, 0.05);
     if (embed_norm_) put("embed.norm", W, 0, 0, 0.05);
     if (pair_buckets_ > 0) put("bigram", (int64_t)pair_buckets_ + 1, W, 0, 1.0);
@@ -584,14 +697,45 @@ bool StackModel::init_synthetic(uint64_t seed) {
     if (L.weights_of >= 0) continue;
     const std::string p = "l" + std::to_string(li) + ".";
     const double sw = 1.0 / sqrt((double)W);
-    if (block_ == 2) {
+    if (block_ == 2 && norm_kind_ == 1) {
+      put_norm(p + "norm1"), put_norm(p + "norm1b");
+      if (L.mlp != 0) put_norm(p + "norm2"), put_norm(p + "norm2b");
+    } else if (block_ == 2) {
       put(p + "norm1", W, 0, 0, 0.05), put(p + "norm1b", W, 0, 0, 0.05);
       if (L.mlp != 0) put(p + "norm2", W, 0, 0, 0.05), put(p + "norm2b", W, 0, 0, 0.05);
     } else {
       put_norm(p + "norm1");
       if (block_ == 1 && L.mlp != 0) put_norm(p + "norm2");
     }
-    if (L.mixer == 3) {
+    if (L.mixer == 3 && !L.lowrank) {
+      const int H = L.heads, nk = L.nk(), nv = H * L.vdim;
+      put(p + "mix.q", nk, W, 0, sw), put(p + "mix.k", nk, W, 0, sw), put(p + "mix.v", nv, W, 0, sw), put(p + "mix.b", H, W, 0, sw);
+      put(p + "mix.q.conv", nk, L.conv, 0.3, 0.3), put(p + "mix.k.conv", nk, L.conv, 0.3, 0.3), put(p + "mix.v.conv", nv, L.conv, 0.3, 0.3);
+      put(p + "mix.a", H, W, 0, sw), put(p + "mix.g", nv, W, 0, sw);
+      put(p + "mix.A_log", H, 0, -1.0, 0.5), put(p + "mix.dt_bias", H, 0, -2.0, 1.0), put(p + "mix.norm", L.vdim, 0, 1, 0.05);
+      put(p + "mix.o", W, nv, 0, 1.0 / sqrt((double)nv));
+    } else if (L.mixer == 6) {
+      const int H = L.heads;
+      put(p + "mix.q", (int64_t)H * L.dim, W, 0, sw), put(p + "mix.k", (int64_t)H * L.dim, W, 0, sw), put(p + "mix.v", (int64_t)H * L.vdim, W, 0, sw);
+      put(p + "mix.g", (int64_t)H * L.vdim, W, 0, sw), put(p + "mix.o", W, H * L.vdim, 0, 1.0 / sqrt((double)H * L.vdim));
+      put(p + "mix.norm", (int64_t)H * L.vdim, 0, 1, 0.05);
+    } else if (L.mixer == 5 && L.right_kind == 1) {
+      const std::string pl = p + "mix.left.", pr = p + "mix.right.";
+      const int H = L.heads, Wr = L.r_width, nb = L.r_blocks, bw = Wr / nb;
+      put(pl + "q", L.nq(), W, 0, sw), put(pl + "k", L.nk(), W, 0, sw), put(pl + "v", L.nv(), W, 0, sw);
+      if (L.has_bias) put(pl + "q.b", L.nq(), 0, 0, 0.02), put(pl + "k.b", L.nk(), 0, 0, 0.02), put(pl + "v.b", L.nv(), 0, 0, 0.02);
+      if (L.qk_norm) put(pl + "q.norm", L.dim, 0, 1, 0.05), put(pl + "k.norm", L.dim, 0, 1, 0.05);
+      if (L.head_temp) put(pl + "temp", H, 0, 1, 0.1);
+      if (L.sink) put(pl + "sink", H, 0, 0, 1.0);
+      if (L.head_gate) put(pl + "g", H, W, 0, sw);
+      put(pl + "o", W, H * L.vdim, 0, 1.0 / sqrt((double)H * L.vdim));
+      put(pr + "y", Wr, W, 0, sw), put(pr + "y.b", Wr, 0, 0, 0.02), put(pr + "x", Wr, W, 0, sw), put(pr + "x.b", Wr, 0, 0, 0.02);
+      put(pr + "conv", Wr, L.conv, 0.3, 0.3), put(pr + "conv.b", Wr, 0, 0, 0.02);
+      put(pr + "ra", (int64_t)nb * bw, bw, 0, 1.0 / sqrt((double)bw)), put(pr + "ri", (int64_t)nb * bw, bw, 0, 1.0 / sqrt((double)bw));
+      put(pr + "ra.b", Wr, 0, 0, 0.1), put(pr + "ri.b", Wr, 0, 0, 0.1), put(pr + "lam", Wr, 0, -2.0, 1.0);
+      put(pr + "o", W, Wr, 0, 1.0 / sqrt((double)Wr));
+      if (L.branch_norm) put(pl + "out", W, 0, 1, 0.05), put(pr + "out", W, 0, 1, 0.05);
+    } else if (L.mixer == 3) {
       const int H = L.heads, nk = L.nk(), nv = H * L.vdim;
       put(p + "mix.q", nk, W, 0, sw), put(p + "mix.k", nk, W, 0, sw), put(p + "mix.v", nv, W, 0, sw), put(p + "mix.b", H, W, 0, sw);
       put(p + "mix.q.conv", nk, L.conv, 0.3, 0.3), put(p + "mix.k.conv", nk, L.conv, 0.3, 0.3), put(p + "mix.v.conv", nv, L.conv, 0.3, 0.3);
@@ -631,7 +775,7 @@ bool StackModel::init_synthetic(uint64_t seed) {
       put(p + "mix.pb", L.heads, 0, -3.0, 0.5), put(p + "mix.talk", L.heads, L.heads, 1.0 / L.heads, 0.1 / L.heads);
     }
     if (L.mixer < 3) put(p + "mix.o", W, L.heads * L.vdim, 0, 1.0 / sqrt((double)L.heads * L.vdim));
-    if (L.mlp == 3) {
+    if (L.mlp == 3 || L.mlp == 4) {
       put(p + "mlp.gate", L.ff, W, 0, sw), put(p + "mlp.up", L.ff, W, 0, sw), put(p + "mlp.down", W, L.ff, 0, 1.0 / sqrt((double)L.ff));
     } else if (L.mlp == 1) {
       put(p + "mlp.up", L.ff, W, 0, sw), put(p + "mlp.down", W, L.ff, 0, 1.0 / sqrt((double)L.ff));
@@ -641,8 +785,9 @@ bool StackModel::init_synthetic(uint64_t seed) {
       a.data.assign((const uint8_t*)c, (const uint8_t*)c + 16);
       staged_[p + "mlp.act"] = a;
     } else if (L.mlp == 2) {
-      put(p + "mlp.router", L.experts, W, 0, sw);
+      put(p + "mlp.router", L.experts + L.n_identity, W, 0, sw);
       if (L.router_kind == 1) put(p + "mlp.router.b", L.experts, 0, 0, 0.1);
+      if (L.router_kind == 2) put(p + "mlp.correction", L.experts + L.n_identity, 0, 0, 0.02);
       for (int e = 0; e < L.experts; e++) {
         const std::string pe = p + "mlp.e" + std::to_string(e) + ".";
         put(pe + "gate", L.ff, W, 0, sw), put(pe + "up", L.ff, W, 0, sw), put(pe + "down", W, L.ff, 0, 1.0 / sqrt((double)L.ff));
@@ -690,8 +835,8 @@ bool StackModel::init_kv_cache(int num_blocks) {
 int64_t StackModel::state_bytes_per_slot() const {
   int64_t b = 0;
   for (const StackLayer& L : layers_) {
-    if (L.s_heads() <= 0) continue;
-    b += (int64_t)L.s_heads() * L.s_dim() * L.s_vdim() * 4;
+    if (L.s_heads() <= 0 && L.vec_state() <= 0) continue;
+    b += (int64_t)L.s_heads() * L.s_dim() * L.s_vdim() * 4 + (int64_t)L.vec_state() * 4;
     if (L.conv > 1) b += (int64_t)(L.conv - 1) * L.conv_channels() * 4;
   }
   return b;
@@ -700,8 +845,8 @@ bool StackModel::init_state(int slots) {
   if (!spec_error_.empty()) return error = spec_error_, false;
   state_slots_ = slots;
   for (StackLayer& L : layers_) {
-    if (L.s_heads() <= 0) continue;
-    const size_t sb = (size_t)slots * L.s_heads() * L.s_dim() * L.s_vdim() * 4;
+    if (L.s_heads() <= 0 && L.vec_state() <= 0) continue;
+    const size_t sb = (size_t)slots * ((size_t)L.s_heads() * L.s_dim() * L.s_vdim() + (size_t)L.vec_state()) * 4;
     if (!(L.state = (float*)dalloc(sb)) || hipMemset(L.state, 0, sb) != hipSuccess) return error = "state slots: allocation failed", false;
     if (L.conv > 1) {
       const size_t cb = (size_t)slots * (L.conv - 1) * L.conv_channels() * 4;
@@ -717,8 +862,21 @@ void StackModel::rotary_table(StackLayer& L) {
   L.rot_pairs = L.rot_dims / 2;
   L.rot_mag = 1.f;
   std::vector<float> fh(std::max(L.rot_pairs, 1), 0.f), fl(std::max(L.rot_pairs, 1), 0.f);
+  // YaRN: pairs that turn fewer than yarn_slow times over the original length are slowed down by the factor, those that turn more than
+  // yarn_fast times are kept, a linear ramp over the pair index between; cos and sin grow by 0.1 ln(factor) + 1
+  double ylo = 0.0, yhi = 0.0;
+  if (L.yarn_factor > 0.0) {
+    const double dims = (double)L.rot_dims, lnb = log(L.rot_base);
+    auto turn_dim = [&](double turns) { return dims * log(L.yarn_original / (2.0 * M_PI * turns)) / (2.0 * lnb); };
+    ylo = std::max(floor(turn_dim(L.yarn_fast)), 0.0), yhi = std::min(ceil(turn_dim(L.yarn_slow)), dims - 1.0);
+    L.rot_mag = (float)(0.1 * log(L.yarn_factor) + 1.0);
+  }
   for (int i = 0; i < L.rot_pairs; i++) {
     double fr = pow(L.rot_base, -2.0 * (double)i / (double)L.rot_dims);
+    if (L.yarn_factor > 0.0) {
+      const double ramp = std::min(std::max(((double)i - ylo) / std::max(yhi - ylo, 0.001), 0.0), 1.0);
+      fr = fr / L.yarn_factor * ramp + fr * (1.0 - ramp);
+    }
     if (L.rs_factor > 0.0) {
       const double wl = 2.0 * M_PI / fr;
       if (wl > L.rs_original / L.rs_low) fr = fr / L.rs_factor;
@@ -738,6 +896,7 @@ bool StackModel::init_buffers(int max_tokens, int max_seqs) {
   const size_t T = max_tokens, W = width_;
   size_t nqkv = 0, nattn = 0, zc = 0, actc = 0, top = 0, experts = 0;
   size_t nqa = 0, z2c = 0, recc = 0, roc = 0;
+  bool want_h32 = false;
   for (const StackLayer& L : layers_) {
     // softmax / sigmoid: the joint projection in the model's type; latent: q, later the heads' values (the joint projection is f32 in z_)
     nqkv = std::max(nqkv, L.mixer == 0 ? (size_t)L.nqkv() : std::max((size_t)L.nq(), (size_t)L.heads * L.vdim));
@@ -746,19 +905,24 @@ bool StackModel::init_buffers(int max_tokens, int max_seqs) {
     if (L.mixer == 1) nqa = std::max(nqa, (size_t)L.heads * (L.kv_rank + L.rot_dim)), actc = std::max(actc, T * L.q_rank);
     if (L.mixer != 0) zc = std::max(zc, T * L.nqkv());
     if (L.mlp == 2) top = std::max(top, (size_t)L.top), experts = std::max(experts, (size_t)L.experts);
-    if (L.mlp == 3) zc = std::max(zc, T * 2 * L.sffp), actc = std::max(actc, T * L.sffp);
-    if (L.mixer >= 3) {  // the joint projection is f32 in z_, the low-rank first stages in act_, their second stages in z2_
+    if (L.mlp == 3 || L.mlp == 4) zc = std::max(zc, T * 2 * L.sffp), actc = std::max(actc, T * L.sffp);
+    if (L.mlp == 2 && L.n_identity > 0) want_h32 = true;
+    if (L.mixer == 5 && L.right_kind == 1) {  // the convolved branch in rec_, both gates' logits in z2_, the recurrence's output in attn_
+      nattn = std::max(nattn, (size_t)L.r_width), z2c = std::max(z2c, (size_t)2 * L.r_width), recc = std::max(recc, (size_t)L.r_width), roc = std::max<size_t>(roc, 1);
+    } else if (L.mixer >= 3) {  // the joint projection is f32 in z_, the low-rank first stages in act_, their second stages in z2_
       const size_t sh = L.s_heads(), sd = L.s_dim(), sv = L.s_vdim();
       nattn = std::max(nattn, sh * sv);
       actc = std::max(actc, T * (size_t)(L.rank_a + L.rank_g));
       z2c = std::max(z2c, sh * sd + (L.mixer == 3 ? sh * sv : 0));
       recc = std::max(recc, L.mixer == 3 ? (size_t)L.conv_channels() + sh + sh * sd : (L.mixer == 4 ? 2 * sh * sd : sh * sd));
+      if (L.mixer == 6) z2c = std::max<size_t>(z2c, 1);
       roc = std::max(roc, sh * sv);
     }
   }
   max_rows_ = (int)round_up((int)(T * std::max<size_t>(top, 1) + experts * 63), 64);
   for (const StackLayer& L : layers_) {
     if (L.mlp == 1) zc = std::max(zc, T * L.ff), actc = std::max(actc, T * L.ff);
+    if (L.mlp == 2 && L.n_identity > 0) experts = std::max(experts, (size_t)L.experts);
     if (L.mlp == 2) {
       zc = std::max(zc, std::max((size_t)max_rows_ * 2 * L.ffp, T * 2 * L.sffp));
       actc = std::max(actc, std::max((size_t)max_rows_ * L.ffp, T * L.sffp));
@@ -782,6 +946,7 @@ bool StackModel::init_buffers(int max_tokens, int max_seqs) {
     sig_scratch_bytes_ = std::max(sig_scratch_bytes_, (size_t)max_seqs * 64 * hv * 4);
   }
   if (sig_scratch_bytes_ && !(sig_scratch_ = (float*)dalloc(sig_scratch_bytes_))) return false;
+  if (want_h32 && (!(h32_ = (float*)dalloc(T * W * 4)) || !(id_weight_ = (float*)dalloc(T * 4)))) return false;
   const size_t P = T * std::max<size_t>(top, 1);
   if (!(pair_expert_ = (int*)dalloc(P * 4)) || !(pair_weight_ = (float*)dalloc(P * 4)) || !(gate_ = (float*)dalloc(T * 4)) ||
       !(row_token_ = (int*)dalloc((size_t)max_rows_ * 4)) || !(row_pair_ = (int*)dalloc((size_t)max_rows_ * 4)) ||
@@ -1070,6 +1235,23 @@ bool StackModel::mixer_delta(const StackLayer& L, const InputMetadata& md, int64
   StkGemmArgs p;
   p.a = h_, p.lda = W, p.w = L.qkv, p.M = T, p.N = n1, p.K = W, p.out = z_, p.ldo = n1, p.out_f32 = 1;
   vra_stack_gemm(p, dt_, stream);
+  if (!L.lowrank) {  // decays (one per head) and gate are columns of the joint projection
+    StkDeltaPrepArgs d;
+    d.raw = z_, d.ld = n1, d.raw2 = z_ + C + H, d.ld2 = n1, d.conv_w = L.conv_w, d.taps = L.conv, d.conv_state = L.conv_state ? L.conv_state : rec_;
+    d.rate = L.rate, d.dt_bias = L.dt_bias, d.q_scale = 1.f / sqrtf((float)D), d.decay_dim = 1;
+    d.qkv_out = rec_, d.beta_out = rec_ + (size_t)T * C, d.decay_out = rec_ + (size_t)T * (C + H);
+    d.positions = md.positions, d.cu_q = md.is_prefill ? md.cu_seqlens_q : nullptr, d.state_slots = md.state_slots;
+    d.T = T, d.B = md.n_seqs, d.H = H, d.G = G, d.dim = D, d.vdim = V;
+    vra_stack_delta_prep(d, stream);
+    vra_stack_conv_state_update(d, stream);
+    StkScanArgs sc;
+    sc.q = rec_, sc.ldq = C, sc.k = rec_ + G * D, sc.ldk = C, sc.v = rec_ + 2 * G * D, sc.ldv = C, sc.qk_rep = H / G;
+    sc.decay = d.decay_out, sc.ldd = H, sc.decay_per_head = 1, sc.beta = d.beta_out, sc.ldb = H;
+    scan_common(sc, L, md, ro_);
+    vra_stack_linear_scan(sc, stream);
+    if (take_stack_err(error, "delta rule")) return false;
+    return recurrent_tail(L, md, z_ + C + 2 * H, n1, 1, L.o, o_, stream);
+  }
   StkGemmArgs l1;
   l1.a = h_, l1.lda = W, l1.w = L.lr1, l1.M = T, l1.N = R, l1.K = W, l1.out = act_, l1.ldo = R;
   vra_stack_gemm(l1, dt_, stream);
@@ -1172,12 +1354,16 @@ bool StackModel::forward_sandwich(const InputMetadata& md, int64_t stream) {
   vra_stack_embed_pair(e, dt_, stream);
   if (take_stack_err(error, "embedding")) return false;
   StkSandwichArgs pend;  // the parts of the last sub-block's output, not yet normed and added (post_w null: none)
-  auto seam = [&](const float* pre_w, const StackLayer* router) {
+  auto seam = [&](const float* pre_w, const float* pre_b, float pre_alpha, const StackLayer* router) {
     StkSandwichArgs s = pend;
-    s.x = x_, s.pre_w = pre_w, s.h = h_, s.eps = eps_, s.T = T, s.W = W;
+    s.x = x_, s.pre_w = pre_w, s.pre_b = pre_b, s.pre_alpha = pre_alpha, s.dyt = norm_kind_ == 1, s.h = h_, s.eps = eps_, s.T = T, s.W = W;
     if (router) {
-      s.router_w = router->router, s.router_bias = router->router_bias, s.n_router = router->experts, s.top = router->top;
+      s.router_w = router->router, s.router_bias = router->router_bias, s.n_router = router->experts + router->n_identity, s.top = router->top;
       s.pair_expert = pair_expert_, s.pair_weight = pair_weight_;
+      if (router->router_kind == 2) {
+        s.router_kind = 1, s.n_groups = router->n_groups, s.keep = router->keep, s.n_identity = router->n_identity;
+        if (router->n_identity > 0) s.h32 = h32_, s.id_weight = id_weight_;
+      }
     }
     if (s.post_w || s.pre_w) vra_stack_sandwich_norm(s, dt_, stream);
     pend = StkSandwichArgs();
@@ -1185,12 +1371,22 @@ bool StackModel::forward_sandwich(const InputMetadata& md, int64_t stream) {
   };
   for (size_t li = 0; li < layers_.size(); li++) {
     const StackLayer& L = layers_[li];
-    if (!seam(L.norm_w, nullptr)) return false;
-    if (!(L.mixer == 3 ? mixer_delta(L, md, stream) : (L.mixer == 4 ? mixer_retention(L, md, stream) : mixer_parallel(L, md, stream)))) return false;
-    pend.p1 = o_, pend.n1 = 1, pend.post_w = L.post1_w;
-    if (L.mixer == 5) pend.c1 = L.left_scale, pend.p2 = sh_, pend.c2 = L.right_scale;
+    if (!seam(L.norm_w, L.norm_b, L.norm_alpha, nullptr)) return false;
+    bool ok = false;
+    switch (L.mixer) {
+      case 3: ok = mixer_delta(L, md, stream); break;
+      case 4: ok = mixer_retention(L, md, stream); break;
+      case 6: ok = mixer_lightning(L, md, stream); break;
+      default: ok = L.right_kind == 1 ? mixer_hybrid(L, md, stream) : mixer_parallel(L, md, stream); break;
+    }
+    if (!ok) return false;
+    pend.p1 = o_, pend.n1 = 1, pend.post_w = L.post1_w, pend.post_b = L.post1_b, pend.post_alpha = L.post1_alpha;
+    if (L.mixer == 5) {
+      pend.c1 = L.left_scale, pend.p2 = sh_, pend.c2 = L.right_scale;
+      if (L.branch_norm) pend.p1_norm_w = L.left_out_w, pend.p2_norm_w = L.right_out_w;
+    }
     if (L.mlp == 2) {
-      if (!seam(L.norm2_w, &L)) return false;
+      if (!seam(L.norm2_w, L.norm2_b, L.norm2_alpha, &L)) return false;
       const int P = T * L.top;
       const int granule = vra_stack_gemm_granule(P, L.experts);
       const int rows = round_up(P + L.experts * (granule - 1), granule);
@@ -1199,17 +1395,96 @@ bool StackModel::forward_sandwich(const InputMetadata& md, int64_t stream) {
       if (take_stack_err(error, "expert rows")) return false;
       // (the weights of a softmax router multiply the experts' OUTPUTS: the rows go in unscaled, the sum over a token's pairs carries them)
       if (!expert_pair(h_, W, L.e_gu, (int64_t)2 * L.ffp * W, L.e_down, (int64_t)W * L.ffp, rows, L.ffp, L.ff, L.limit, tile_group_, granule, row_token_,
-                       L.router_kind == 1 ? nullptr : row_scale_, row_pair_, pair_out_, stream, L.act_kind))
+                       L.router_kind >= 1 ? nullptr : row_scale_, row_pair_, pair_out_, stream, L.act_kind))
         return false;
-      pend.p1 = pair_out_, pend.n1 = L.top, pend.pw = L.router_kind == 1 ? pair_weight_ : nullptr, pend.post_w = L.post2_w;
+      pend.p1 = pair_out_, pend.n1 = L.top, pend.pw = L.router_kind >= 1 ? pair_weight_ : nullptr;
+      pend.post_w = L.post2_w, pend.post_b = L.post2_b, pend.post_alpha = L.post2_alpha;
+      if (L.router_kind == 2 && L.n_identity > 0) {  // an identity expert's pair has no row: its weight times the feed-forward's own input
+        pend.pe = pair_expert_, pend.p2 = h32_, pend.p2w = id_weight_, pend.c2 = 1.f;
+      }
+    } else if (L.mlp == 4) {
+      if (!seam(L.norm2_w, L.norm2_b, L.norm2_alpha, nullptr)) return false;
+      if (!expert_pair(h_, W, L.s_gu, 0, L.s_down, 0, T, L.sffp, L.ff, L.limit, nullptr, 0, nullptr, nullptr, nullptr, pair_out_, stream, 0)) return false;
+      pend.p1 = pair_out_, pend.n1 = 1, pend.post_w = L.post2_w, pend.post_b = L.post2_b, pend.post_alpha = L.post2_alpha;
     }
     if (trace_on_ || li + 1 == layers_.size()) {
-      if (!seam(nullptr, nullptr)) return false;
+      if (!seam(nullptr, nullptr, 1.f, nullptr)) return false;
       if (trace_on_ && hipMemcpyAsync(trace_ + li * (size_t)T * W, x_, (size_t)T * W * 4, hipMemcpyDeviceToDevice, st) != hipSuccess)
         return error = "layer trace copy failed", false;
     }
   }
   return true;
+}
+
+// lightning: q | k | v | gate in one launch (f32); q, k, v pass silu on their way into the recurrence (one constant decay per head);
+// one norm over the concatenated heads, sigmoid gate, output projection
+bool StackModel::mixer_lightning(const StackLayer& L, const InputMetadata& md, int64_t stream) {
+  const int T = md.n_tokens, W = width_, H = L.heads, D = L.dim, V = L.vdim, n1 = L.nqkv();
+  StkGemmArgs p;
+  p.a = h_, p.lda = W, p.w = L.qkv, p.M = T, p.N = n1, p.K = W, p.out = z_, p.ldo = n1, p.out_f32 = 1;
+  vra_stack_gemm(p, dt_, stream);
+  StkScanArgs sc;
+  sc.q = z_, sc.ldq = n1, sc.k = z_ + H * D, sc.ldk = n1, sc.v = z_ + 2 * H * D, sc.ldv = n1, sc.head_decay = L.head_decay, sc.act_silu = 1;
+  scan_common(sc, L, md, ro_);
+  vra_stack_linear_scan(sc, stream);
+  if (take_stack_err(error, "lightning")) return false;
+  vra_stack_head_norm_gate(ro_, L.out_norm_w, z_ + 2 * H * D + H * V, n1, 2, eps_, attn_, T, 1, H * V, dt_, stream);
+  StkGemmArgs o;
+  o.a = attn_, o.lda = H * V, o.w = L.o, o.M = T, o.N = W, o.K = H * V, o.out = o_, o.ldo = W, o.out_f32 = 1;
+  vra_stack_gemm(o, dt_, stream);
+  return !take_stack_err(error, "lightning");
+}
+
+// two branches on one input, each with a norm of its own in the seam that follows.  Left: softmax attention over the paged cache (biases
+// in the projection's epilogue; per-head q / k norm and rotary on neighbouring pairs in the launch that writes the cache rows; sliding
+// window, sink, per-head temperature and the per-head sigmoid output gate inside the attention) -> o_.  Right: gelu branch times a
+// real-gated diagonal recurrence behind a short convolution; its gates are block-diagonal products in f32 -> sh_.
+bool StackModel::mixer_hybrid(const StackLayer& L, const InputMetadata& md, int64_t stream) {
+  const int T = md.n_tokens, B = md.n_seqs, W = width_, n1 = L.nqkv(), H = L.heads, Wr = L.r_width, nb = L.r_blocks, bw = Wr / nb;
+  const int lq = L.nq(), lk = L.nk(), lv = L.nv(), g0 = lq + lk + lv, y0 = g0 + (L.head_gate ? H : 0), x0 = y0 + Wr;
+  StkGemmArgs p;
+  p.a = h_, p.lda = W, p.w = L.qkv, p.bias = L.qkv_bias, p.M = T, p.N = n1, p.K = W, p.out = z_, p.ldo = n1, p.out_f32 = 1;
+  vra_stack_gemm(p, dt_, stream);
+  // left
+  StkHeadPrepArgs hp;
+  hp.raw = z_, hp.ld = n1, hp.q_off = 0, hp.k_off = lq, hp.v_off = lq + lk, hp.Hq = H, hp.Hk = L.kv_heads, hp.dim = L.dim, hp.nv = lv;
+  hp.qn_w = L.qn_w, hp.kn_w = L.kn_w, hp.eps = eps_;
+  hp.rot.freq_hi = L.freq_hi, hp.rot.freq_lo = L.freq_lo, hp.rot.pairs = L.rot_pairs, hp.rot.mag = L.rot_mag, hp.rot_pairs_layout = L.rot_layout;
+  hp.positions = md.positions, hp.q_out = qkv_, hp.q_ld = lq, hp.k_out = kc_[L.cache], hp.k_ld = lk, hp.v_out = vc_[L.cache], hp.v_ld = lv;
+  hp.slots = md.slot_mapping, hp.T = T;
+  vra_stack_head_prep(hp, dt_, stream);
+  StkAttnArgs a;
+  a.q = qkv_, a.ldq = lq, a.out = attn_, a.kc = kc_[L.cache], a.vc = vc_[L.cache];
+  a.positions = md.positions, a.block_tables = md.block_tables, a.context_lens = md.context_lens;
+  a.cu_q = md.is_prefill ? md.cu_seqlens_q : nullptr;
+  a.B = B, a.T = T, a.max_q = md.is_prefill ? md.max_seqlen_q : 1, a.H = H, a.G = L.kv_heads, a.dim = L.dim, a.vdim = L.vdim;
+  a.BS = ec_.block_size, a.max_blocks = md.max_blocks, a.scale = L.scale, a.chunk = L.chunk, a.window = L.window;
+  a.sink = L.sink ? L.sink_w : nullptr, a.head_scale = L.head_temp ? L.temp_w : nullptr;
+  if (L.head_gate) a.gate = z_ + g0, a.gate_ld = n1;
+  vra_stack_attention(a, dt_, stream);
+  StkGemmArgs o;
+  o.a = attn_, o.lda = H * L.vdim, o.w = L.o, o.M = T, o.N = W, o.K = H * L.vdim, o.out = o_, o.ldo = W, o.out_f32 = 1;
+  vra_stack_gemm(o, dt_, stream);
+  if (take_stack_err(error, "parallel mixer (attention)")) return false;
+  // right
+  StkConvArgs cv;
+  cv.x = z_ + x0, cv.ld = n1, cv.C = Wr, cv.taps = L.conv, cv.w = L.conv_w, cv.bias = L.conv_b, cv.conv_state = L.conv_state, cv.y = rec_, cv.ldy = Wr;
+  cv.positions = md.positions, cv.cu_q = md.is_prefill ? md.cu_seqlens_q : nullptr, cv.state_slots = md.state_slots, cv.T = T, cv.B = B;
+  vra_stack_conv_rows(cv, stream);
+  vra_stack_conv_rows_update(cv, stream);
+  StkGemmArgs g;  // per block: [T, bw] x [2 bw, bw]^T -> both gates' logits, f32 whatever the model's type
+  g.a = rec_, g.lda = Wr, g.a_batch_stride = bw, g.w = L.gates_w, g.w_batch_stride = (int64_t)2 * bw * bw, g.batch = nb;
+  g.bias = L.gates_b, g.bias_batch_stride = 2 * bw, g.M = T, g.N = 2 * bw, g.K = bw, g.out = z2_, g.ldo = 2 * Wr, g.out_batch_stride = 2 * bw, g.out_f32 = 1;
+  vra_stack_gemm(g, VRA_F32, stream);
+  StkGatedScanArgs gs;
+  gs.u = rec_, gs.ldu = Wr, gs.gr = z2_, gs.gi = z2_ + bw, gs.ldg = 2 * Wr, gs.y = z_ + y0, gs.ldy = n1, gs.lam = L.lam, gs.rate = 8.f;
+  gs.state = L.state, gs.state_slots = md.state_slots, gs.positions = md.positions, gs.cu_q = cv.cu_q, gs.out = attn_, gs.ldo = Wr, gs.B = B, gs.C = Wr;
+  gs.block = bw;
+  vra_stack_gated_scan(gs, dt_, stream);
+  StkGemmArgs ro;
+  ro.a = attn_, ro.lda = Wr, ro.w = L.r_o, ro.M = T, ro.N = W, ro.K = Wr, ro.out = sh_, ro.ldo = W, ro.out_f32 = 1;
+  vra_stack_gemm(ro, dt_, stream);
+  return !take_stack_err(error, "parallel mixer (gated recurrence)");
 }
 
 int64_t StackModel::read_layer_trace(void* host, int64_t max_bytes, int64_t stream) {

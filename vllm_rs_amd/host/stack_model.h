@@ -21,7 +21,18 @@
 //                      with wavelength-dependent scaling, visibility inside blocks of `chunk` positions) and a gated linear attention
 //                      (decay per key channel sigmoid(z)^(1 / tau) from a low-rank projection)
 //           delta, retention and the right branch keep a matrix state [dim, vdim] per head and sequence (f32, one slot per live sequence)
+//           lightning: linear attention with a constant decay per head, q / k / v through silu, no rotation, ONE norm over the concatenated
+//                      heads, sigmoid gate
+//           delta with lowrank=0: one decay per head and token, decay and silu gate projected at full rank (no low-rank stages)
+//           parallel with right=rglru: the left branch's softmax attention sees a sliding window, has a sink per head, a temperature per
+//                      head, a sigmoid output gate per head and rotary on neighbouring pairs (YaRN-scaled); the right branch is a gelu branch
+//                      times a real-gated diagonal recurrence behind a short convolution (block-diagonal gates); each branch's output has an
+//                      RMS norm of its own over the width (branch_norm=1) before the scaled sum
 //   mlp     none | dense (PolyNorm activation) | moe (sigmoid router, clamped gated experts, gated shared expert) | gated (gelu_tanh(gate) * up)
+//           | clamped (dense, the clamped gated form of the experts above);  moe with router=softmax_all: scores are a softmax over all
+//           router outputs, a correction is added for the choice only, the choice is restricted to the best `keep` of `groups` groups of
+//           neighbouring experts, the weights are the plain scores, and the last `identity` outputs are experts that return their input
+//   sandwich blocks with norm=dyt use Dynamic Tanh for all four norms of a layer; tie_head=1: the head is the embedding table
 //   weights_of=j: the layer runs with layer j's tensors and a cache of its own
 // vllm_rs_amd/checkpoint.py turns a design's config.json into the spec text below.
 //
@@ -35,7 +46,9 @@
 //         window=.. keep_first=.. slope_exp=..
 //         conv=.. rank_a=.. rank_g=.. decay=d0,d1,.. chunk=.. qk_norm=0|1 bias=0|1 rs_factor=.. rs_low=.. rs_high=.. rs_original=..
 //         r_heads=.. r_dim=.. r_vdim=.. tau=.. left_scale=.. right_scale=..
-//         mlp=none|dense|moe|gated ff=.. experts=.. top=.. limit=.. shared_ff=.. shared_limit=.. router=sigmoid|softmax act=clamped|silu
+//         lowrank=0|1 right=gla|rglru r_width=.. r_blocks=.. r_conv=.. head_temp=0|1 head_gate=0|1 rot_layout=half|pairs branch_norm=0|1
+//         mlp=none|dense|moe|gated|clamped ff=.. experts=.. top=.. limit=.. shared_ff=.. shared_limit=.. router=sigmoid|softmax|softmax_all
+//         act=clamped|silu identity=.. groups=.. keep=..
 #pragma once
 #include <map>
 #include <string>
@@ -47,7 +60,7 @@ namespace vra {
 
 struct StackLayer {
   // mixer: 0 softmax attention, 1 latent attention, 2 sigmoid attention, 3 gated delta rule, 4 retention, 5 parallel (softmax attention
-  // beside a gated linear attention)
+  // beside a gated linear attention or a real-gated diagonal recurrence), 6 lightning
   int mixer = 0;
   int heads = 0, kv_heads = 0, dim = 0, vdim = 0, temp_every = 0, kv_from = -1, weights_of = -1;
   float scale = 1.f, softcap = 0.f, temp_coef = 0.f;
@@ -65,7 +78,13 @@ struct StackLayer {
   double rs_factor = 0.0, rs_low = 1.0, rs_high = 4.0, rs_original = 0.0;
   int r_heads = 0, r_dim = 0, r_vdim = 0;
   float tau = 1.f, left_scale = 1.f, right_scale = 1.f;
-  // feed-forward: 0 none, 1 dense (PolyNorm), 2 mixture of experts, 3 gated dense (gelu_tanh(gate) * up)
+  // delta: lowrank 0 = decay (one per head) and gate come from the joint projection.  parallel: right_kind 1 = real-gated diagonal recurrence
+  // of r_width channels with r_blocks gate blocks behind a convolution of `conv` taps; the left branch's per-head temperature and output
+  // gate, rotary layout (1 = neighbouring pairs), a norm per branch before the sum
+  int lowrank = 1, right_kind = 0, r_width = 0, r_blocks = 1, head_temp = 0, head_gate = 0, rot_layout = 0, branch_norm = 0;
+  // router_kind 2: identity experts and expert groups
+  int n_identity = 0, n_groups = 0, keep = 0;
+  // feed-forward: 0 none, 1 dense (PolyNorm), 2 mixture of experts, 3 gated dense (gelu_tanh(gate) * up), 4 clamped gated dense
   int mlp = 0, ff = 0, experts = 0, top = 0, shared_ff = 0;
   float limit = 0.f, shared_limit = 0.f;
   // mixture of experts: router 0 = sigmoid scores as weights on the experts' inputs, 1 = biased logits, softmax over the chosen ones, weights
@@ -82,17 +101,19 @@ struct StackLayer {
   int nqkv() const {
     if (mixer == 1) return q_rank + kv_rank + rot_dim;
     if (mixer == 2) return nq() + nk() + nv() + heads * vdim;
-    if (mixer == 3) return 2 * nk() + heads * vdim + heads;          // q | k (kv_heads each) | v | write strengths
-    if (mixer == 4) return 2 * heads * dim + 2 * heads * vdim;       // q | k | v | gate
+    if (mixer == 3) return 2 * nk() + heads * vdim + heads + (lowrank ? 0 : heads + heads * vdim);  // q | k (kv_heads each) | v | write strengths (| decays | gate)
+    if (mixer == 4 || mixer == 6) return 2 * heads * dim + 2 * heads * vdim;       // q | k | v | gate
+    if (mixer == 5 && right_kind == 1) return nq() + nk() + nv() + (head_gate ? heads : 0) + 2 * r_width;  // left q | k | v | gates, right gelu branch | recurrent branch
     if (mixer == 5) return nq() + nk() + nv() + r_heads * (2 * r_dim + 2 * r_vdim);  // left q | k | v, right q | k | v | gate
     return nq() + (owns_cache ? nk() + nv() : 0);
   }
-  bool has_cache() const { return mixer != 3 && mixer != 4; }
+  bool has_cache() const { return mixer != 3 && mixer != 4 && mixer != 6; }
   // the recurrent part: heads, key and value sizes of the matrix state (0 heads: none)
-  int s_heads() const { return mixer == 5 ? r_heads : (mixer == 3 || mixer == 4 ? heads : 0); }
+  int s_heads() const { return mixer == 5 ? (right_kind == 1 ? 0 : r_heads) : (mixer == 3 || mixer == 4 || mixer == 6 ? heads : 0); }
+  int vec_state() const { return mixer == 5 && right_kind == 1 ? r_width : 0; }  // a diagonal recurrence: one state value per channel
   int s_dim() const { return mixer == 5 ? r_dim : dim; }
   int s_vdim() const { return mixer == 5 ? r_vdim : vdim; }
-  int conv_channels() const { return mixer == 3 ? 2 * nk() + heads * vdim : 0; }
+  int conv_channels() const { return mixer == 3 ? 2 * nk() + heads * vdim : vec_state(); }
   // elements of one token's cache rows
   int k_row() const { return mixer == 1 ? kv_rank + rot_dim : nk(); }
   int v_row() const { return mixer == 1 ? 0 : nv(); }
@@ -127,7 +148,11 @@ struct StackLayer {
   float* lr2_bias = nullptr;
   float *conv_w = nullptr, *rate = nullptr, *dt_bias = nullptr, *out_norm_w = nullptr, *head_decay = nullptr;
   void* r_o = nullptr;          // right branch: [width, r_heads * r_vdim]
-  float* state = nullptr;       // [slots, heads, vdim, dim]
+  float *post1_b = nullptr, *post2_b = nullptr;  // Dynamic Tanh in sandwich blocks: offsets and slopes of the output norms
+  float post1_alpha = 1.f, post2_alpha = 1.f;
+  float *temp_w = nullptr, *left_out_w = nullptr, *right_out_w = nullptr;
+  float *conv_b = nullptr, *gates_w = nullptr, *gates_b = nullptr, *lam = nullptr;  // gates_w f32 [r_blocks][2 * bw][bw]: recurrence gate rows, then input gate rows
+  float* state = nullptr;       // [slots, heads, vdim, dim];  a diagonal recurrence: [slots, r_width]
   float* conv_state = nullptr;  // [slots, conv - 1, conv_channels()]
 };
 
@@ -178,6 +203,8 @@ class StackModel : public ModelBase {
   bool mixer_delta(const StackLayer& L, const InputMetadata& md, int64_t stream);
   bool mixer_retention(const StackLayer& L, const InputMetadata& md, int64_t stream);
   bool mixer_parallel(const StackLayer& L, const InputMetadata& md, int64_t stream);
+  bool mixer_lightning(const StackLayer& L, const InputMetadata& md, int64_t stream);
+  bool mixer_hybrid(const StackLayer& L, const InputMetadata& md, int64_t stream);
   bool recurrent_tail(const StackLayer& L, const InputMetadata& md, const float* gate, int gate_ld, int gate_act, const void* w_o, float* out, int64_t stream);
   bool forward_sandwich(const InputMetadata& md, int64_t stream);
   void rotary_table(StackLayer& L);
@@ -194,7 +221,8 @@ class StackModel : public ModelBase {
   int width_ = 0, vocab_ = 0, groups_ = 1;
   int block_ = 0, norm_kind_ = 0, pos_kind_ = 0;  // 0 parallel / rms / sinusoid, 1 sequential / dyt / none, block 2 sandwich
   float norm_offset_ = 0.f, embed_scale_ = 1.f;    // added to every norm weight at load; multiplies the embedding row
-  int embed_norm_ = 0, pair_buckets_ = 0;
+  int embed_norm_ = 0, pair_buckets_ = 0, tie_head_ = 0;
+  float *h32_ = nullptr, *id_weight_ = nullptr;  // identity experts: the unrounded feed-forward input and the summed weight of a token's identity picks
   int64_t pair_mul_prev_ = 0, pair_mul_cur_ = 0;
   void* pair_table_ = nullptr;
   float* embed_norm_w_ = nullptr;
