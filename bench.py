@@ -47,7 +47,7 @@ def parse():
     ap.add_argument("--no-graph", action="store_true", help="eager launches (rocprofv3 kernel tracing crashes on hipGraph replay)")
     ap.add_argument("--blocks", type=int, default=8192, help="KV blocks (64 tokens each); 0 = kv_fraction of free HBM")
     ap.add_argument("--tp", type=int, default=0, help="run ONE tensor-parallel engine over this many ranks (spawns its own runner processes)")
-    ap.add_argument("--design", default="", help="'ditilix', 'gaperax' or 'zifetar': prefill / decode throughput of that layer-stack design beside the dense "
+    ap.add_argument("--design", default="", help="'ditilix', 'gaperax', 'zifetar' or 'sudosun': prefill / decode throughput of that layer-stack design beside the dense "
                     "Llama of the same widths (vllm_rs_amd/stack_bench.py) instead of the default workload")
     return ap.parse_args()
 
@@ -727,10 +727,11 @@ def tp_main(a):
 def main():
     a = parse()
     if a.design:
-        if a.design.lower() not in ("ditilix", "gaperax", "zifetar"):
-            raise SystemExit(f"bench.py: unknown --design {a.design!r} (ditilix, gaperax, zifetar)")
+        if a.design.lower() not in ("ditilix", "gaperax", "zifetar", "sudosun"):
+            raise SystemExit(f"bench.py: unknown --design {a.design!r} (ditilix, gaperax, zifetar, sudosun)")
         from vllm_rs_amd import stack_bench
-        sizes = {"ditilix": stack_bench.SIZES, "gaperax": stack_bench.GAPERAX_SIZES, "zifetar": stack_bench.ZIFETAR_SIZES}[a.design.lower()]
+        sizes = {"ditilix": stack_bench.SIZES, "gaperax": stack_bench.GAPERAX_SIZES, "zifetar": stack_bench.ZIFETAR_SIZES,
+                 "sudosun": stack_bench.SUDOSUN_SIZES}[a.design.lower()]
         stack_bench.main(steps=min(a.steps, 64), warmup=min(a.warmup, 8), graph=not a.no_graph, design=a.design.lower(),
                          sizes=[a.model] if a.model in sizes else None)  # --model <size name>: that size alone
         return 0

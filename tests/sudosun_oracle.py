@@ -84,6 +84,39 @@ def rotate_pairs(x, cos, sin):
 
 
 # ------------------------------------------------------------------------------------------------ mixers
+def constant_decay_recurrence(q, k, v, decay):
+    """q, k [T, H, D], v [T, H, V]: per head S <- decay_h S + k v^T, o = S^T q (the read-out sees the current token's write)"""
+    T, H, D = q.shape
+    o = np.zeros((T, H, v.shape[-1]))
+    for hd in range(H):
+        S = np.zeros((D, v.shape[-1]))
+        for t in range(T):
+            S = decay[hd] * S + np.outer(k[t, hd], v[t, hd])
+            o[t, hd] = S.T @ q[t, hd]
+    return o
+
+
+def delta_rule_recurrence(q, k, v, beta, g):
+    """q, k [T, G, D], v [T, H, V], beta, g [T, H]: S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q"""
+    T, G, D = q.shape
+    H, V = v.shape[1], v.shape[2]
+    o = np.zeros((T, H, V))
+    rep = H // G
+    for hd in range(H):
+        S = np.zeros((D, V))
+        for t in range(T):
+            kt, qt = k[t, hd // rep], q[t, hd // rep]
+            S = g[t, hd] * S
+            u = beta[t, hd] * (v[t, hd] - S.T @ kt)
+            S = S + np.outer(kt, u)
+            o[t, hd] = S.T @ qt
+    return o
+
+
+def unit(x):
+    return x / np.sqrt(np.sum(x * x, -1, keepdims=True) + 1e-6)
+
+
 def mixer_lightning(h, mx, w, p, eps):
     """linear attention with one constant decay per head: S <- d S + k v^T, o = S^T q; q, k, v through silu"""
     T = h.shape[0]
@@ -91,13 +124,7 @@ def mixer_lightning(h, mx, w, p, eps):
     q = silu(h @ w[p + "q"].T).reshape(T, H, D)
     k = silu(h @ w[p + "k"].T).reshape(T, H, D)
     v = silu(h @ w[p + "v"].T).reshape(T, H, V)
-    decay = [float(d) for d in mx["decay"]]
-    o = np.zeros((T, H, V))
-    for hd in range(H):
-        S = np.zeros((D, V))
-        for t in range(T):
-            S = decay[hd] * S + np.outer(k[t, hd], v[t, hd])
-            o[t, hd] = S.T @ q[t, hd]
+    o = constant_decay_recurrence(q, k, v, [float(d) for d in mx["decay"]])
     o = rms(o.reshape(T, H * V), eps) * w[p + "norm"]
     o = o * sigmoid(h @ w[p + "g"].T)
     return o @ w[p + "o"].T
@@ -110,23 +137,33 @@ def mixer_delta(h, mx, w, p, eps):
     q = silu(causal_conv(h @ w[p + "q"].T, w[p + "q.conv"])).reshape(T, G, D)
     k = silu(causal_conv(h @ w[p + "k"].T, w[p + "k.conv"])).reshape(T, G, D)
     v = silu(causal_conv(h @ w[p + "v"].T, w[p + "v.conv"])).reshape(T, H, V)
-    q = q / np.sqrt(np.sum(q * q, -1, keepdims=True) + 1e-6) * D ** -0.5
-    k = k / np.sqrt(np.sum(k * k, -1, keepdims=True) + 1e-6)
+    q, k = unit(q) * D ** -0.5, unit(k)
     beta = sigmoid(h @ w[p + "b"].T)
     g = np.exp(-np.exp(w[p + "A_log"]) * softplus(h @ w[p + "a"].T + w[p + "dt_bias"]))
-    o = np.zeros((T, H, V))
-    rep = H // G
-    for hd in range(H):
-        S = np.zeros((D, V))
-        for t in range(T):
-            kt, qt = k[t, hd // rep], q[t, hd // rep]
-            S = g[t, hd] * S
-            u = beta[t, hd] * (v[t, hd] - S.T @ kt)
-            S = S + np.outer(kt, u)
-            o[t, hd] = S.T @ qt
-    o = rms(o, eps) * w[p + "norm"]
+    o = rms(delta_rule_recurrence(q, k, v, beta, g), eps) * w[p + "norm"]
     o = o.reshape(T, H * V) * silu(h @ w[p + "g"].T)
     return o @ w[p + "o"].T
+
+
+def window_visible(positions, window):
+    """[T, T]: query i sees key j iff 0 <= p_i - p_j < window (window 0: every earlier key)"""
+    pos = np.asarray(positions)
+    dist = pos[:, None] - pos[None, :]
+    return (dist >= 0) & ((dist < window) if window > 0 else True)
+
+
+def softmax_window_sink(q, k, v, head_scale, sink, vis):
+    """q [T, H, D], k [T, G, D], v [T, G, V]: scores q . k times head_scale[h]; the denominator also holds exp(sink[h]), which has no value"""
+    T, H, _ = q.shape
+    G = k.shape[1]
+    out = np.zeros((T, H, v.shape[-1]))
+    for hd in range(H):
+        g = hd // (H // G)
+        s = np.where(vis, (q[:, hd] @ k[:, g].T) * head_scale[hd], -np.inf)
+        m = np.maximum(s.max(-1), sink[hd])
+        e = np.exp(s - m[:, None])
+        out[:, hd] = (e / (e.sum(-1) + np.exp(sink[hd] - m))[:, None]) @ v[:, g]
+    return out
 
 
 def attention_window_sink(h, mx, w, p, eps, positions):
@@ -143,21 +180,20 @@ def attention_window_sink(h, mx, w, p, eps, positions):
         cos, sin = rotary_table(rot, positions)
         q, k = rotate_pairs(q, cos, sin), rotate_pairs(k, cos, sin)
     window = int((mx.get("mask") or {}).get("size", 0))
-    pos = np.asarray(positions)
-    dist = pos[:, None] - pos[None, :]
-    vis = (dist >= 0) & ((dist < window) if window > 0 else True)
-    gate = sigmoid(h @ w[p + "g"].T)  # [T, H]
-    out = np.zeros((T, H, V))
-    rep = H // G
-    for hd in range(H):
-        s = (q[:, hd] @ k[:, hd // rep].T) * float(mx["scale"]) * w[p + "temp"][hd]
-        s = np.where(vis, s, -np.inf)
-        sink = w[p + "sink"][hd]
-        m = np.maximum(s.max(-1), sink)
-        e = np.exp(s - m[:, None])
-        den = e.sum(-1) + np.exp(sink - m)
-        out[:, hd] = (e / den[:, None]) @ v[:, hd // rep] * gate[:, hd:hd + 1]
+    out = softmax_window_sink(q, k, v, float(mx["scale"]) * w[p + "temp"], w[p + "sink"], window_visible(positions, window))
+    out = out * sigmoid(h @ w[p + "g"].T)[:, :, None]  # one gate per head
     return out.reshape(T, H * V) @ w[p + "o"].T
+
+
+def gated_diagonal_recurrence(u, r, i, lam):
+    """u, r, i [T, C]: a = exp(-8 r softplus(lam)); S <- a S + sqrt(1 - a^2) i u from S = 0, the first token included"""
+    a = np.exp(-8.0 * r * softplus(lam))
+    S = np.zeros(u.shape[1])
+    out = np.zeros_like(u)
+    for t in range(u.shape[0]):
+        S = a[t] * S + np.sqrt(1.0 - a[t] ** 2) * i[t] * u[t]
+        out[t] = S
+    return out
 
 
 def gated_linear_unit(h, mx, w, p):
@@ -171,13 +207,7 @@ def gated_linear_unit(h, mx, w, p):
     ub = u.reshape(T, nb, bw)
     r = sigmoid(np.einsum("tbi,boi->tbo", ub, w[p + "ra"]) + w[p + "ra.b"]).reshape(T, C)
     i = sigmoid(np.einsum("tbi,boi->tbo", ub, w[p + "ri"]) + w[p + "ri.b"]).reshape(T, C)
-    a = np.exp(-8.0 * r * softplus(w[p + "lam"]))
-    S = np.zeros(C)
-    out = np.zeros((T, C))
-    for t in range(T):
-        S = a[t] * S + np.sqrt(1.0 - a[t] ** 2) * i[t] * u[t]
-        out[t] = S
-    return (out * y) @ w[p + "o"].T
+    return (gated_diagonal_recurrence(u, r, i, w[p + "lam"]) * y) @ w[p + "o"].T
 
 
 def mixer_parallel(h, mx, w, p, eps, positions):
@@ -234,6 +264,7 @@ def ff_moe(h, mlp, w, p):
 def forward(cfg, w, tokens, return_layers=False):
     """-> logits [T, vocab] (and the residual stream after every layer [L, T, width])"""
     eps = float(cfg["norm"]["eps"])
+    w = {k: np.asarray(v, np.float64) for k, v in w.items()}
     tokens = np.asarray(tokens)
     positions = np.arange(len(tokens))
     x = w["embed"][tokens]
@@ -266,3 +297,89 @@ def greedy(cfg, w, prompt, n):
     for _ in range(n):
         toks.append(int(np.argmax(forward(cfg, w, toks)[-1])))
     return toks[len(prompt):]
+
+
+# ------------------------------------------------------------------------------------------------ random models for the tests
+def bf16_round(a):
+    """float32 array rounded to bfloat16 (nearest even), returned as float32"""
+    u = np.ascontiguousarray(a, np.float32).view(np.uint32).astype(np.uint64)
+    return (((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16).astype(np.uint32).view(np.float32).reshape(np.shape(a))
+
+
+def tensor_shapes(cfg):
+    W = int(cfg["width"])
+    out = {"embed": (int(cfg["vocab"]), W)}
+
+    def norm(name):
+        out[name], out[name + ".b"], out[name + ".alpha"] = (W,), (W,), ()
+    norm("final.norm")
+    for li, layer in enumerate(cfg["layers"]):
+        p, mx = "l%d." % li, layer["mixer"]
+        norm(p + "norm1"), norm(p + "norm1b")
+        if layer.get("mlp"):
+            norm(p + "norm2"), norm(p + "norm2b")
+        m = p + "mix."
+        if layer["type"] == "delta":
+            H, G, D, V, K = int(mx["heads"]), int(mx.get("kv_heads", mx["heads"])), int(mx["dim"]), int(mx.get("vdim", mx["dim"])), int(mx.get("conv", 1))
+            out.update({m + "q": (G * D, W), m + "q.conv": (G * D, K), m + "k": (G * D, W), m + "k.conv": (G * D, K), m + "v": (H * V, W),
+                        m + "v.conv": (H * V, K), m + "b": (H, W), m + "a": (H, W), m + "A_log": (H,), m + "dt_bias": (H,), m + "norm": (V,),
+                        m + "g": (H * V, W), m + "o": (W, H * V)})
+        elif layer["type"] == "lightning":
+            H, D, V = int(mx["heads"]), int(mx["dim"]), int(mx.get("vdim", mx["dim"]))
+            out.update({m + "q": (H * D, W), m + "k": (H * D, W), m + "v": (H * V, W), m + "g": (H * V, W), m + "o": (W, H * V), m + "norm": (H * V,)})
+        else:
+            le, ri = mx["left"], mx["right"]
+            H, G, D, V = int(le["heads"]), int(le.get("kv_heads", le["heads"])), int(le["dim"]), int(le.get("vdim", le["dim"]))
+            C, nb, K = int(ri["width"]), int(ri["blocks"]), int(ri.get("conv", 1))
+            a, b = m + "left.", m + "right."
+            out.update({a + "q": (H * D, W), a + "q.b": (H * D,), a + "k": (G * D, W), a + "k.b": (G * D,), a + "v": (G * V, W), a + "v.b": (G * V,),
+                        a + "q.norm": (D,), a + "k.norm": (D,), a + "temp": (H,), a + "sink": (H,), a + "g": (H, W), a + "o": (W, H * V), a + "out": (W,),
+                        b + "y": (C, W), b + "y.b": (C,), b + "x": (C, W), b + "x.b": (C,), b + "conv": (C, K), b + "conv.b": (C,),
+                        b + "ra": (nb, C // nb, C // nb), b + "ra.b": (nb, C // nb), b + "ri": (nb, C // nb, C // nb), b + "ri.b": (nb, C // nb),
+                        b + "lam": (C,), b + "o": (W, C), b + "out": (W,)})
+        mlp = layer.get("mlp")
+        f = p + "mlp."
+        if mlp and mlp["kind"] == "dense":
+            out.update({f + "gate": (int(mlp["ff"]), W), f + "up": (int(mlp["ff"]), W), f + "down": (W, int(mlp["ff"]))})
+        elif mlp:
+            r, ff = mlp["router"], int(mlp["expert"]["ff"])
+            n = int(r["experts"]) + int(r.get("identity", 0))
+            out.update({f + "router": (n, W), f + "correction": (n,)})
+            for e in range(int(r["experts"])):
+                out.update({"%se%d.gate" % (f, e): (ff, W), "%se%d.up" % (f, e): (ff, W), "%se%d.down" % (f, e): (W, ff)})
+    return out
+
+
+def random_tensors(cfg, seed):
+    """bfloat16-representable float32 tensors: projections ~ N(0, 1.5 / sqrt(fan in)), norm weights around one with slopes below one, decay
+    inputs spread so that some channels forget within a few tokens and others keep hundreds"""
+    r = np.random.default_rng(seed)
+    out = {}
+    for name, shape in tensor_shapes(cfg).items():
+        last = name.split(".")[-1]
+        if last == "alpha":
+            a = 0.3 + 0.5 * r.random(shape)
+        elif last in ("norm1", "norm1b", "norm2", "norm2b", "norm", "out", "temp") or name == "final.norm":
+            a = 1.0 + 0.2 * r.standard_normal(shape)
+        elif last == "dt_bias":
+            a = -2.0 + 1.5 * r.standard_normal(shape)
+        elif last == "A_log":
+            a = -1.0 + 0.7 * r.standard_normal(shape)
+        elif last == "lam":
+            a = -3.0 + 1.5 * r.standard_normal(shape)
+        elif last == "sink":
+            a = r.standard_normal(shape)
+        elif last == "correction":
+            a = 0.05 * r.standard_normal(shape)
+        elif last == "b" and (len(shape) == 1 or name.endswith(("ra.b", "ri.b"))):
+            a = 0.3 * r.standard_normal(shape)
+        elif last == "conv":
+            a = 0.4 * r.standard_normal(shape) + 0.3
+        elif name == "embed":
+            a = r.standard_normal(shape)
+        elif last == "router":
+            a = 3.0 * r.standard_normal(shape) / math.sqrt(shape[-1])
+        else:
+            a = 1.5 * r.standard_normal(shape) / math.sqrt(shape[-1])
+        out[name] = bf16_round(np.asarray(a, np.float32))
+    return out

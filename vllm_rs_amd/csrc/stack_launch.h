@@ -383,7 +383,8 @@ void vra_stack_conv_rows_update(const StkConvArgs& a, int64_t stream);
 // Real-gated diagonal recurrence over a sequence's tokens, one state value per channel (f32 [slots, C]):
 //   r = sigmoid(gr[t, c]), i = sigmoid(gi[t, c]), a = exp(-rate * r * softplus(lam[c])),  S <- a S + sqrt(1 - a^2) (i u[t, c]),
 //   out[t, c] = S * gelu_tanh(y[t, c])  in dtype.
-// Tokens run in order; a sequence whose first row stands at position 0 starts from S = 0.
+// Tokens run in order; a sequence whose first row stands at position 0 starts from S = 0.  T = rows of the step.  A prompt step (cu_q)
+// OVERWRITES gr, gi and y with the decay, the weighted input and the activated branch.
 struct StkGatedScanArgs {
   const float* u = nullptr;
   int ldu = 0;
@@ -403,4 +404,4 @@ struct StkGatedScanArgs {
   int ldo = 0;
   int B = 0, C = 0;
 };
-void vra_stack_gated_scan(const StkGatedScanArgs& a, int dtype, int64_t stream);
+void vra_stack_gated_scan(const StkGatedScanArgs& a, int T, int dtype, int64_t stream);

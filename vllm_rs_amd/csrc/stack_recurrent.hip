@@ -601,12 +601,34 @@ __global__ __launch_bounds__(256) void stk_conv_rows_update_kernel(StkConvArgs a
 }
 
 // ------------------------------------------------------------------------------------------------ real-gated diagonal recurrence
-// lane = channel, a sequence's tokens in order.  The operands of GT tokens are requested together and a tile ahead; gates, decay and input
-// weight of a tile are formed before its GT dependent multiply-adds run, so only those wait for one another.
+// Two forms.  One token per sequence: one launch forms gates, decay and input weight and moves the state on.  Prompt portions: an
+// element-wise launch over all tokens and channels first turns the gate logits into the decay a and the weighted input b IN PLACE (and the
+// gelu branch into its activation), so that the launch that walks a sequence's tokens in order has one multiply-add per token and three
+// operands to fetch — requested two tiles ahead, since nothing in them depends on the state.
 __device__ __forceinline__ float gelu_tanhf_(float z) {
   return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
 }
-template <typename T>
+// (a, b) of one token and channel: a = exp(-sl r), b = sqrt(1 - a^2) i u with 1 - a^2 = -expm1(2 ln a) (no cancellation near a = 1)
+__device__ __forceinline__ void gated_coef(float sl, float gr, float gi, float u, float* a, float* b) {
+  const float la = -sl * sigmoidf_(gr);
+  *a = expf(la);
+  *b = sqrtf(-expm1f(2.f * la)) * (sigmoidf_(gi) * u);
+}
+__global__ __launch_bounds__(256) void stk_gated_prep_kernel(StkGatedScanArgs a, int T) {
+  const int64_t total = (int64_t)T * a.C;
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total; e += (int64_t)gridDim.x * 256) {
+    const int64_t t = e / a.C;
+    const int c = (int)(e % a.C);
+    const int gc = a.block > 0 ? c / a.block * 2 * a.block + c % a.block : c;
+    float* gr = const_cast<float*>(a.gr) + t * a.ldg + gc;
+    float* gi = const_cast<float*>(a.gi) + t * a.ldg + gc;
+    float* y = const_cast<float*>(a.y) + t * a.ldy + c;
+    float av, bv;
+    gated_coef(a.rate * softplusf_(a.lam[c]), *gr, *gi, a.u[t * a.ldu + c], &av, &bv);
+    *gr = av, *gi = bv, *y = gelu_tanhf_(*y);
+  }
+}
+template <typename T, bool PREPARED>
 __global__ __launch_bounds__(64) void stk_gated_scan_kernel(StkGatedScanArgs a) {
   constexpr int GT = 8;
   const int b = blockIdx.y, c = blockIdx.x * 64 + threadIdx.x;
@@ -616,35 +638,47 @@ __global__ __launch_bounds__(64) void stk_gated_scan_kernel(StkGatedScanArgs a) 
   const bool fresh = a.positions[t0] == 0;
   float* sp = a.state + (size_t)slot * a.C + c;
   float S = fresh ? 0.f : *sp;
-  const float sl = a.rate * softplusf_(a.lam[c]);
   const int gc = a.block > 0 ? c / a.block * 2 * a.block + c % a.block : c;
   T* out = (T*)a.out;
-  float un[GT], rn[GT], in_[GT], yn[GT];
-  auto request = [&](int i0) {
+  if (!PREPARED) {
+    const float sl = a.rate * softplusf_(a.lam[c]);
+    for (int i = 0; i < n; i++) {
+      const size_t t = (size_t)(t0 + i);
+      float av, bv;
+      gated_coef(sl, a.gr[t * a.ldg + gc], a.gi[t * a.ldg + gc], a.u[t * a.ldu + c], &av, &bv);
+      S = fmaf(av, S, bv);
+      El<T>::st(out + t * a.ldo + c, S * gelu_tanhf_(a.y[t * a.ldy + c]));
+    }
+    *sp = S;
+    return;
+  }
+  float av[3][GT], bv[3][GT], yv[3][GT];  // three tiles of operands: one in use, two on their way
+  auto request = [&](int i0, int w) {
 #pragma unroll
     for (int j = 0; j < GT; j++) {
       const size_t t = (size_t)(t0 + min(i0 + j, n - 1));
-      un[j] = a.u[t * a.ldu + c], rn[j] = a.gr[t * a.ldg + gc], in_[j] = a.gi[t * a.ldg + gc], yn[j] = a.y[t * a.ldy + c];
+      av[w][j] = a.gr[t * a.ldg + gc], bv[w][j] = a.gi[t * a.ldg + gc], yv[w][j] = a.y[t * a.ldy + c];
     }
   };
-  request(0);
-  for (int i0 = 0; i0 < n; i0 += GT) {
-    float av[GT], bv[GT], yv[GT];
+  auto run = [&](int i0, int w) {
 #pragma unroll
-    for (int j = 0; j < GT; j++) {
-      const float la = -sl * sigmoidf_(rn[j]), aj = expf(la);
-      av[j] = aj;
-      bv[j] = sqrtf(-expm1f(2.f * la)) * (sigmoidf_(in_[j]) * un[j]);  // (1 - a^2 without the cancellation near a = 1)
-      yv[j] = gelu_tanhf_(yn[j]);
-    }
-    if (i0 + GT < n) request(i0 + GT);
-#pragma unroll
-    for (int j = 0; j < GT; j++) {
+    for (int j = 0; j < GT; j++)
       if (i0 + j < n) {
-        S = fmaf(av[j], S, bv[j]);
-        El<T>::st(out + (size_t)(t0 + i0 + j) * a.ldo + c, S * yv[j]);
+        S = fmaf(av[w][j], S, bv[w][j]);
+        El<T>::st(out + (size_t)(t0 + i0 + j) * a.ldo + c, S * yv[w][j]);
       }
-    }
+  };
+  request(0, 0);
+  if (GT < n) request(GT, 1);
+  for (int i0 = 0; i0 < n; i0 += 3 * GT) {  // (the tile index is a compile-time constant in every call: the operands stay in registers)
+    if (i0 + 2 * GT < n) request(i0 + 2 * GT, 2);
+    run(i0, 0);
+    if (i0 + GT >= n) break;
+    if (i0 + 3 * GT < n) request(i0 + 3 * GT, 0);
+    run(i0 + GT, 1);
+    if (i0 + 2 * GT >= n) break;
+    if (i0 + 4 * GT < n) request(i0 + 4 * GT, 1);
+    run(i0 + 2 * GT, 2);
   }
   *sp = S;
 }
@@ -766,12 +800,21 @@ void vra_stack_conv_rows_update(const StkConvArgs& a, int64_t stream) {
   const dim3 grid(a.B, std::min((a.C + 255) / 256, 64));
   launch_checked("stack convolution state", [&] { stk_conv_rows_update_kernel<<<grid, 256, 0, as_stream(stream)>>>(a); });
 }
-void vra_stack_gated_scan(const StkGatedScanArgs& a, int dtype, int64_t stream) {
+void vra_stack_gated_scan(const StkGatedScanArgs& a, int T, int dtype, int64_t stream) {
   VRA_CHECK_ARG(a.u && a.gr && a.gi && a.y && a.lam && a.state && a.state_slots && a.positions && a.out, "stack gated scan: null pointer");
   VRA_CHECK_ARG(a.B > 0 && a.C > 0 && a.ldu >= a.C && a.ldy >= a.C && a.ldo >= a.C, "stack gated scan: shapes");
   const dim3 grid((a.C + 63) / 64, a.B);
-  if (dtype == VRA_F32) launch_checked("stack gated scan", [&] { stk_gated_scan_kernel<float><<<grid, 64, 0, as_stream(stream)>>>(a); });
-  else launch_checked("stack gated scan", [&] { stk_gated_scan_kernel<uint16_t><<<grid, 64, 0, as_stream(stream)>>>(a); });
+  hipStream_t st = as_stream(stream);
+  if (!a.cu_q) {
+    if (dtype == VRA_F32) launch_checked("stack gated scan", [&] { stk_gated_scan_kernel<float, false><<<grid, 64, 0, st>>>(a); });
+    else launch_checked("stack gated scan", [&] { stk_gated_scan_kernel<uint16_t, false><<<grid, 64, 0, st>>>(a); });
+    return;
+  }
+  VRA_CHECK_ARG(T > 0, "stack gated scan: a prompt step names its rows");
+  const int pg = (int)std::min<int64_t>(((int64_t)T * a.C + 255) / 256, 8192);
+  launch_checked("stack gated scan (gates)", [&] { stk_gated_prep_kernel<<<pg, 256, 0, st>>>(a, T); });
+  if (dtype == VRA_F32) launch_checked("stack gated scan", [&] { stk_gated_scan_kernel<float, true><<<grid, 64, 0, st>>>(a); });
+  else launch_checked("stack gated scan", [&] { stk_gated_scan_kernel<uint16_t, true><<<grid, 64, 0, st>>>(a); });
 }
 
 // ================================================================================================ C entry points (operator tests)

@@ -1480,7 +1480,7 @@ bool StackModel::mixer_hybrid(const StackLayer& L, const InputMetadata& md, int6
   gs.u = rec_, gs.ldu = Wr, gs.gr = z2_, gs.gi = z2_ + bw, gs.ldg = 2 * Wr, gs.y = z_ + y0, gs.ldy = n1, gs.lam = L.lam, gs.rate = 8.f;
   gs.state = L.state, gs.state_slots = md.state_slots, gs.positions = md.positions, gs.cu_q = cv.cu_q, gs.out = attn_, gs.ldo = Wr, gs.B = B, gs.C = Wr;
   gs.block = bw;
-  vra_stack_gated_scan(gs, dt_, stream);
+  vra_stack_gated_scan(gs, T, dt_, stream);
   StkGemmArgs ro;
   ro.a = attn_, ro.lda = Wr, ro.w = L.r_o, ro.M = T, ro.N = W, ro.K = Wr, ro.out = sh_, ro.ldo = W, ro.out_f32 = 1;
   vra_stack_gemm(ro, dt_, stream);

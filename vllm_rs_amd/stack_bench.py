@@ -1,5 +1,6 @@
-"""Throughput of a layer-stack model (Ditilix, Gaperax or Zifetar design) beside the dense bf16 Llama of the same widths —
-`python bench.py --design ditilix|gaperax|zifetar` (Zifetar also beside the Ditilix mixture of experts of the same widths, the closest
+"""Throughput of a layer-stack model (Ditilix, Gaperax, Zifetar or Sudosun design) beside the dense bf16 Llama of the same widths —
+`python bench.py --design ditilix|gaperax|zifetar|sudosun` (Sudosun also beside the Zifetar design of the same widths, its closest model;
+Zifetar also beside the Ditilix mixture of experts of the same widths, the closest
 model of its class).
 
 Random weights of layer sizes that resemble a real model; for each size one JSON line with prefill tokens/s (one prompt of
@@ -112,6 +113,44 @@ def zifetar_costs(cj):
     return 2 * n, 2 * n
 
 
+def sudosun_config(width, heads, kv_heads, dim, layers, vocab, experts, top, expert_ff, window, blocks):
+    """config.json dict of a Sudosun model: layers in the order parallel, delta rule, lightning, ...; every layer a mixture of experts (four
+    identity experts beside the real ones, four groups of which two may be chosen from)"""
+    rot = dict(base=1e6, dims=dim // 2, scaling=dict(factor=8.0, original=4096, fast=16.0, slow=2.0))
+    par = dict(left=dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim, scale=dim ** -0.5, mask=dict(size=window), rot=rot),
+               right=dict(width=width, blocks=blocks, conv=4))
+    dl = dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim, conv=4)
+    li = dict(heads=heads, dim=dim, vdim=dim, decay=[1.0 - 2.0 ** (-5.0 - 5.0 * h / max(heads - 1, 1)) for h in range(heads)])
+    mlp = dict(kind="moe", expert=dict(ff=expert_ff), router=dict(experts=experts, top=top, identity=4, groups=dict(count=4, keep=2)))
+    kinds = [("parallel", par), ("delta", dl), ("lightning", li)]
+    ls = [dict(type=kinds[i % 3][0], mixer=kinds[i % 3][1], mlp=mlp) for i in range(layers)]
+    return dict(architecture="Sudosun", width=width, vocab=vocab, norm=dict(eps=1e-6), logit_scale=1.0, layers=ls)
+
+
+def sudosun_costs(cj):
+    """(matrix FLOPs per token without attention and recurrences, weight bytes a one-token step reads) of a Sudosun config"""
+    W, n = cj["width"], 0
+    for layer in cj["layers"]:
+        mx = layer["mixer"]
+        if layer["type"] == "parallel":
+            le, ri = mx["left"], mx["right"]
+            H, G, D, V, Wr = le["heads"], le["kv_heads"], le["dim"], le["vdim"], ri["width"]
+            n += W * (H * D + G * D + G * V + H + 2 * Wr) + 2 * Wr * (Wr // ri["blocks"]) + (H * V + Wr) * W
+        elif layer["type"] == "delta":
+            H, G, D, V = mx["heads"], mx["kv_heads"], mx["dim"], mx["vdim"]
+            n += W * (2 * G * D + 2 * H * V + 2 * H) + H * V * W
+        else:
+            H, D, V = mx["heads"], mx["dim"], mx["vdim"]
+            n += W * (2 * H * D + 2 * H * V) + H * V * W
+        mlp = layer.get("mlp")
+        if mlp and mlp["kind"] == "moe":
+            n += mlp["router"]["top"] * 3 * W * mlp["expert"]["ff"] + W * (mlp["router"]["experts"] + mlp["router"].get("identity", 0))
+        elif mlp:
+            n += 3 * W * mlp["ff"]
+    n += cj["vocab"] * W
+    return 2 * n, 2 * n
+
+
 def llama_costs(cfg):
     H, D = cfg["hidden_size"], cfg["head_dim"]
     per = H * (cfg["num_heads"] + 2 * cfg["num_kv_heads"]) * D + cfg["num_heads"] * D * H + 3 * H * cfg["intermediate_size"]
@@ -175,14 +214,25 @@ ZIFETAR_SIZES = {
 }
 
 
+SUDOSUN_SIZES = {
+    # name: (width, heads, kv_heads, head size, layers, vocab, experts, top, expert ff, window, gate blocks of the recurrence)
+    "sudosun-2048": (2048, 16, 4, 128, 3, 32000, 16, 2, 1024, 1024, 16),
+    "sudosun-4096": (4096, 32, 8, 128, 3, 32000, 16, 2, 2048, 1024, 32),
+}
+
+
 def main(steps=64, warmup=8, prefill_tokens=2048, graph=True, sizes=None, design="ditilix"):
     from . import _lib, checkpoint
     from .engine import BF16, Engine
     L = _lib.load()
     lines = []
-    table = GAPERAX_SIZES if design == "gaperax" else (ZIFETAR_SIZES if design == "zifetar" else SIZES)
+    table = GAPERAX_SIZES if design == "gaperax" else (ZIFETAR_SIZES if design == "zifetar" else (SUDOSUN_SIZES if design == "sudosun" else SIZES))
     for name in (sizes or table):
-        if design == "zifetar":
+        if design == "sudosun":
+            width, heads, kvh, dim, layers, vocab, experts, top, eff, window, blocks = table[name]
+            cj = sudosun_config(width, heads, kvh, dim, layers, vocab, experts, top, eff, window, blocks)
+            ff = 4 * width
+        elif design == "zifetar":
             width, heads, kvh, dim, layers, vocab, experts, top, eff, chunk, rank = table[name]
             cj = zifetar_config(width, heads, kvh, dim, layers, vocab, experts, top, eff, chunk, rank)
             ff = 4 * width
@@ -196,7 +246,13 @@ def main(steps=64, warmup=8, prefill_tokens=2048, graph=True, sizes=None, design
         res = dict(stack=measure(eng, L, vocab, prefill_tokens, steps, warmup))
         eng.close()
         res["stack"]["flops_per_token"], res["stack"]["weight_bytes_per_step"] = (
-            zifetar_costs(cj) if design == "zifetar" else (gaperax_costs(cj) if design == "gaperax" else stack_costs(cj)))
+            sudosun_costs(cj) if design == "sudosun" else (zifetar_costs(cj) if design == "zifetar" else (gaperax_costs(cj) if design == "gaperax" else stack_costs(cj))))
+        if design == "sudosun":  # the closest model of the same class: the Zifetar design of the same widths (state mixers, the same experts)
+            zj = zifetar_config(width, heads, kvh, dim, layers, vocab, experts, top, eff, window, width // 32)
+            eng = Engine(checkpoint.parse_config(zj), num_gpu_blocks=512, max_num_seqs=8, max_model_len=4096, use_graph=graph).init_synthetic()
+            res["zifetar"] = measure(eng, L, vocab, prefill_tokens, steps, warmup)
+            eng.close()
+            res["zifetar"]["flops_per_token"], res["zifetar"]["weight_bytes_per_step"] = zifetar_costs(zj)
         if design == "zifetar":  # the closest model of the same class: softmax attention + the same mixture of experts in every layer
             dj = stack_config(width, heads, kvh, dim, ff, layers + 1, vocab, experts, top, eff, 0, False)
             dj["layers"] = dj["layers"][1:]
@@ -213,7 +269,7 @@ def main(steps=64, warmup=8, prefill_tokens=2048, graph=True, sizes=None, design
         for m in res.values():
             m["prefill_matrix_tflops"] = m["prefill_tokens_per_s"] * m["flops_per_token"] / 1e12
             m["decode_bs1_weight_gb_per_s"] = m["weight_bytes_per_step"] / (m["decode_bs1_ms_per_step"] / 1e3) / 1e9
-        line = dict(metric="stack_vs_dense_llama", size=name, design={"gaperax": "Gaperax", "zifetar": "Zifetar"}.get(design, "Ditilix"), dtype="bf16", data="synthetic", prefill_tokens=prefill_tokens,
+        line = dict(metric="stack_vs_dense_llama", size=name, design={"gaperax": "Gaperax", "zifetar": "Zifetar", "sudosun": "Sudosun"}.get(design, "Ditilix"), dtype="bf16", data="synthetic", prefill_tokens=prefill_tokens,
                     decode_context=512, steps=steps, **res)
         print(json.dumps(line), flush=True)
         lines.append(line)
