@@ -701,6 +701,39 @@ void vra_stack_op_sandwich_norm(float* x, const float* p1, int32_t n1, const flo
                                 const float* router_bias, int32_t n_router, int32_t top, int32_t* pair_expert, float* pair_weight,
                                 int32_t dtype, int64_t stream);
 
+/* attention_window: the softmax attention under a sliding window (key j visible iff 0 <= p_i - j < window; 0 = causal), with a sink per head
+ * in the denominator, a scale per head on the scores and sigmoid(gate[t, h]) on head h's output row (null pointers: absent).
+ * seam: vra_stack_op_sandwich_norm with Dynamic Tanh norms (dyt = 1: tanh(alpha v) w + b), an RMS norm of its own per part (p1_norm_w /
+ * p2_norm_w), pairs without a row (pe < 0), a per-row weight on the second part (p2w), the unrounded h (h32), and router_kind 1: softmax
+ * over all n_router outputs, router_bias added for the choice only, choice within the `keep` best of n_groups groups, weights = scores,
+ * the last n_identity outputs chosen as expert -1 with their weights summed into id_weight.
+ * conv_rows: y = act(bias + causal convolution per channel over a sequence's rows, the inputs before the step from conv_state), then
+ * the state moves on.  gated_scan: S <- a S + sqrt(1 - a^2) sigmoid(gi) u, a = exp(-rate sigmoid(gr) softplus(lam)); out = S gelu_tanh(y);
+ * a prompt step (cu_q) overwrites gr, gi, y.  linear_scan_ex: vra_stack_op_linear_scan with one decay per head and token
+ * (decay_per_head) or silu on q, k, v (act_silu). */
+void vra_stack_op_attention_window(const void* q, int32_t ldq, void* out, const void* kc, const void* vc, const int64_t* positions,
+                                   const uint32_t* block_tables, const uint32_t* context_lens, const uint32_t* cu_q, int32_t B, int32_t T,
+                                   int32_t max_q, int32_t H, int32_t G, int32_t dim, int32_t vdim, int32_t BS, int32_t max_blocks,
+                                   float scale, int32_t window, const float* sink, const float* head_scale, const float* gate,
+                                   int32_t gate_ld, int32_t dtype, int64_t stream);
+void vra_stack_op_seam(float* x, const float* p1, int32_t n1, const float* pw, const int32_t* pe, float c1, const float* p2, const float* p2w,
+                       float c2, const float* p1_norm_w, const float* p2_norm_w, int32_t dyt, const float* post_w, const float* post_b,
+                       float post_alpha, const float* pre_w, const float* pre_b, float pre_alpha, void* h, float* h32, float eps, int32_t T,
+                       int32_t W, const void* router_w, const float* router_bias, int32_t router_kind, int32_t n_router, int32_t top,
+                       int32_t n_groups, int32_t keep, int32_t n_identity, int32_t* pair_expert, float* pair_weight, float* id_weight,
+                       int32_t dtype, int64_t stream);
+void vra_stack_op_conv_rows(const float* x, int32_t ld, int32_t C, int32_t taps, const float* w, const float* bias, float* conv_state,
+                            int32_t act, float* y, int32_t ldy, const int64_t* positions, const uint32_t* cu_q, const int32_t* state_slots,
+                            int32_t T, int32_t B, int64_t stream);
+void vra_stack_op_gated_scan(const float* u, int32_t ldu, float* gr, float* gi, int32_t ldg, int32_t block, float* y, int32_t ldy,
+                             const float* lam, float rate, float* state, const int32_t* state_slots, const int64_t* positions,
+                             const uint32_t* cu_q, void* out, int32_t ldo, int32_t B, int32_t C, int32_t T, int32_t dtype, int64_t stream);
+void vra_stack_op_linear_scan_ex(const float* q, int32_t ldq, const float* k, int32_t ldk, const float* v, int32_t ldv, const float* decay,
+                                 int32_t ldd, int32_t decay_per_head, int32_t act_silu, const float* head_decay, const float* beta,
+                                 int32_t ldb, float q_scale, float* state, const int32_t* state_slots, const int64_t* positions,
+                                 const uint32_t* cu_q, float* out, int32_t ldo, int32_t B, int32_t H, int32_t qk_rep, int32_t dim,
+                                 int32_t vdim, int64_t stream);
+
 /* decode-step microbenchmark hook used by bench.py: runs `steps` decode steps of the current
  * running batch back to back (graph replay when enabled) and returns elapsed ms measured with HIP
  * events on the engine stream; tokens are sampled and appended exactly as in vra_engine_step. */

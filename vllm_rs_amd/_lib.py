@@ -221,6 +221,14 @@ def load():
     _sig(lib, "vra_stack_op_linear_scan", None, P, c_i32, P, c_i32, P, c_i32, P, c_i32, P, P, c_i32, c_f32, P, P, P, P, P, c_i32, c_i32, c_i32, c_i32,
          c_i32, c_i32, c_i64)
     _sig(lib, "vra_stack_op_sandwich_norm", None, P, P, c_i32, P, c_f32, P, c_f32, P, P, P, c_f32, c_i32, c_i32, P, P, c_i32, c_i32, P, P, c_i32, c_i64)
+    _sig(lib, "vra_stack_op_attention_window", None, P, c_i32, P, P, P, P, P, P, P, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32,
+         c_f32, c_i32, P, P, P, c_i32, c_i32, c_i64)
+    _sig(lib, "vra_stack_op_seam", None, P, P, c_i32, P, P, c_f32, P, P, c_f32, P, P, c_i32, P, P, c_f32, P, P, c_f32, P, P, c_f32, c_i32, c_i32, P, P,
+         c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, P, P, P, c_i32, c_i64)
+    _sig(lib, "vra_stack_op_conv_rows", None, P, c_i32, c_i32, c_i32, P, P, P, c_i32, P, c_i32, P, P, P, c_i32, c_i32, c_i64)
+    _sig(lib, "vra_stack_op_gated_scan", None, P, c_i32, P, P, c_i32, c_i32, P, c_i32, P, c_f32, P, P, P, P, P, c_i32, c_i32, c_i32, c_i32, c_i32, c_i64)
+    _sig(lib, "vra_stack_op_linear_scan_ex", None, P, c_i32, P, c_i32, P, c_i32, P, c_i32, c_i32, c_i32, P, P, c_i32, c_f32, P, P, P, P, P, c_i32, c_i32,
+         c_i32, c_i32, c_i32, c_i32, c_i64)
     _sig(lib, "vra_engine_create_spec", P, MC, EC, C.c_char_p)
     _sig(lib, "vra_engine_replay_step", c_i32, P, c_i32, P, P, P, P, P, c_i32, P, P)
     _sig(lib, "vra_engine_debug_layer_trace", None, P, c_i32)

@@ -846,3 +846,60 @@ extern "C" void vra_stack_op_sandwich_norm(float* x, const float* p1, int32_t n1
   a.router_w = router_w, a.router_bias = router_bias, a.n_router = n_router, a.top = top, a.pair_expert = pair_expert, a.pair_weight = pair_weight;
   vra_stack_sandwich_norm(a, dtype, stream);
 }
+
+// the softmax attention with a sliding window, a sink, a scale per head and a sigmoid output gate per head
+extern "C" void vra_stack_op_attention_window(const void* q, int32_t ldq, void* out, const void* kc, const void* vc, const int64_t* positions,
+                                              const uint32_t* block_tables, const uint32_t* context_lens, const uint32_t* cu_q, int32_t B, int32_t T,
+                                              int32_t max_q, int32_t H, int32_t G, int32_t dim, int32_t vdim, int32_t BS, int32_t max_blocks, float scale,
+                                              int32_t window, const float* sink, const float* head_scale, const float* gate, int32_t gate_ld,
+                                              int32_t dtype, int64_t stream) {
+  StkAttnArgs a;
+  a.q = q, a.ldq = ldq, a.out = out, a.kc = kc, a.vc = vc, a.positions = positions, a.block_tables = block_tables, a.context_lens = context_lens;
+  a.cu_q = cu_q, a.B = B, a.T = T, a.max_q = max_q, a.H = H, a.G = G, a.dim = dim, a.vdim = vdim, a.BS = BS, a.max_blocks = max_blocks;
+  a.scale = scale, a.window = window, a.sink = sink, a.head_scale = head_scale, a.gate = gate, a.gate_ld = gate_ld;
+  vra_stack_attention(a, dtype, stream);
+}
+// the seam with Dynamic Tanh norms, per-branch norms, pairs without a row, a weighted second part and the router over all outputs
+extern "C" void vra_stack_op_seam(float* x, const float* p1, int32_t n1, const float* pw, const int32_t* pe, float c1, const float* p2, const float* p2w,
+                                  float c2, const float* p1_norm_w, const float* p2_norm_w, int32_t dyt, const float* post_w, const float* post_b,
+                                  float post_alpha, const float* pre_w, const float* pre_b, float pre_alpha, void* h, float* h32, float eps, int32_t T,
+                                  int32_t W, const void* router_w, const float* router_bias, int32_t router_kind, int32_t n_router, int32_t top,
+                                  int32_t n_groups, int32_t keep, int32_t n_identity, int32_t* pair_expert, float* pair_weight, float* id_weight,
+                                  int32_t dtype, int64_t stream) {
+  StkSandwichArgs a;
+  a.x = x, a.p1 = p1, a.n1 = n1, a.pw = pw, a.pe = pe, a.c1 = c1, a.p2 = p2, a.p2w = p2w, a.c2 = c2, a.p1_norm_w = p1_norm_w, a.p2_norm_w = p2_norm_w;
+  a.dyt = dyt, a.post_w = post_w, a.post_b = post_b, a.post_alpha = post_alpha, a.pre_w = pre_w, a.pre_b = pre_b, a.pre_alpha = pre_alpha;
+  a.h = h, a.h32 = h32, a.eps = eps, a.T = T, a.W = W, a.router_w = router_w, a.router_bias = router_bias, a.router_kind = router_kind;
+  a.n_router = n_router, a.top = top, a.n_groups = n_groups, a.keep = keep, a.n_identity = n_identity;
+  a.pair_expert = pair_expert, a.pair_weight = pair_weight, a.id_weight = id_weight;
+  vra_stack_sandwich_norm(a, dtype, stream);
+}
+// short causal convolution with its state (rows, then the state's update) and the real-gated diagonal recurrence
+extern "C" void vra_stack_op_conv_rows(const float* x, int32_t ld, int32_t C, int32_t taps, const float* w, const float* bias, float* conv_state,
+                                       int32_t act, float* y, int32_t ldy, const int64_t* positions, const uint32_t* cu_q, const int32_t* state_slots,
+                                       int32_t T, int32_t B, int64_t stream) {
+  StkConvArgs a;
+  a.x = x, a.ld = ld, a.C = C, a.taps = taps, a.w = w, a.bias = bias, a.conv_state = conv_state, a.act = act, a.y = y, a.ldy = ldy;
+  a.positions = positions, a.cu_q = cu_q, a.state_slots = state_slots, a.T = T, a.B = B;
+  vra_stack_conv_rows(a, stream);
+  vra_stack_conv_rows_update(a, stream);
+}
+extern "C" void vra_stack_op_gated_scan(const float* u, int32_t ldu, float* gr, float* gi, int32_t ldg, int32_t block, float* y, int32_t ldy,
+                                        const float* lam, float rate, float* state, const int32_t* state_slots, const int64_t* positions,
+                                        const uint32_t* cu_q, void* out, int32_t ldo, int32_t B, int32_t C, int32_t T, int32_t dtype, int64_t stream) {
+  StkGatedScanArgs a;
+  a.u = u, a.ldu = ldu, a.gr = gr, a.gi = gi, a.ldg = ldg, a.block = block, a.y = y, a.ldy = ldy, a.lam = lam, a.rate = rate, a.state = state;
+  a.state_slots = state_slots, a.positions = positions, a.cu_q = cu_q, a.out = out, a.ldo = ldo, a.B = B, a.C = C;
+  vra_stack_gated_scan(a, T, dtype, stream);
+}
+// the linear recurrence with one decay per head and token (delta rule) or silu on q, k, v (constant decays)
+extern "C" void vra_stack_op_linear_scan_ex(const float* q, int32_t ldq, const float* k, int32_t ldk, const float* v, int32_t ldv, const float* decay,
+                                            int32_t ldd, int32_t decay_per_head, int32_t act_silu, const float* head_decay, const float* beta, int32_t ldb,
+                                            float q_scale, float* state, const int32_t* state_slots, const int64_t* positions, const uint32_t* cu_q,
+                                            float* out, int32_t ldo, int32_t B, int32_t H, int32_t qk_rep, int32_t dim, int32_t vdim, int64_t stream) {
+  StkScanArgs a;
+  a.q = q, a.ldq = ldq, a.k = k, a.ldk = ldk, a.v = v, a.ldv = ldv, a.decay = decay, a.ldd = ldd, a.decay_per_head = decay_per_head, a.act_silu = act_silu;
+  a.head_decay = head_decay, a.beta = beta, a.ldb = ldb, a.q_scale = q_scale, a.state = state, a.state_slots = state_slots, a.positions = positions;
+  a.cu_q = cu_q, a.out = out, a.ldo = ldo, a.B = B, a.H = H, a.qk_rep = qk_rep, a.dim = dim, a.vdim = vdim;
+  vra_stack_linear_scan(a, stream);
+}
