@@ -90,7 +90,7 @@ def test_native_parser_accepts_the_layer_list():
     (lambda s: s.replace("rot_layout=pairs", "rot_layout=thirds", 1), "rot_layout half or pairs"),
     (lambda s: s.replace("groups=3 keep=2", "groups=4 keep=2"), "groups must divide"),
     (lambda s: s.replace("groups=3 keep=2", "groups=3 keep=4"), "keep <= groups"),
-    (lambda s: s.replace("router=softmax_all", "router=dice", 1), "router is sigmoid, softmax or softmax_all"),
+    (lambda s: s.replace("router=softmax_all", "router=dice", 1), "router is sigmoid or softmax or softmax_all"),
     (lambda s: s.replace("mlp=clamped ff=28", "mlp=clamped ff=0"), "without ff"),
     (lambda s: s.replace("mixer=lightning", "mixer=thunder"), "unknown mixer"),
 ])

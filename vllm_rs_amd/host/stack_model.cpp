@@ -92,7 +92,7 @@ bool StackModel::parse_spec(const char* spec) {
       {
         const std::string rk = f.count("router") ? f["router"] : "sigmoid", ak = f.count("act") ? f["act"] : "clamped";
         if ((rk != "sigmoid" && rk != "softmax" && rk != "softmax_all") || (ak != "clamped" && ak != "silu"))
-          return spec_error_ = "layer stack spec: router is sigmoid, softmax or softmax_all, act clamped or silu", false;
+          return spec_error_ = "layer stack spec: router is sigmoid or softmax or softmax_all, act clamped or silu", false;
         L.router_kind = rk == "softmax" ? 1 : (rk == "softmax_all" ? 2 : 0), L.act_kind = ak == "silu" ? 2 : 0;
         L.n_identity = (int)num("identity", 0), L.n_groups = (int)num("groups", 0), L.keep = (int)num("keep", 0);
       }
