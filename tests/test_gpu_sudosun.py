@@ -410,6 +410,27 @@ def test_greedy_generation_through_the_scheduler(use_graph):
         assert len(out) == 12
 
 
+def test_sampled_generation_stays_inside_the_top_k():
+    """the framework's sampler on this design's logits (temperature, top-k 3): every sampled token is one of the three most likely by the
+    oracle's logits for the sequence so far (or within rounding of the third), and a penalised run still finishes"""
+    cfg = config_a()
+    tensors = so.random_tensors(cfg, 21)
+    eng = build(cfg, tensors, F32, blocks=16, max_model_len=256, num_state_slots=2)
+    prompts = [tokens_of(cfg, n, 80 + n) for n in (9, 40)]
+    outs = eng.generate(prompts, max_tokens=8, ignore_eos=True, sampling=dict(temperature=0.9, top_k=3, top_p=1.0))
+    pen = eng.generate(prompts[:1], max_tokens=6, ignore_eos=True, sampling=dict(temperature=0.7, top_k=4, top_p=0.9, frequency_penalty=0.5, presence_penalty=0.2))
+    eng.close()
+    assert len(pen[0]) == 6
+    for p, out in zip(prompts, outs):
+        seq = list(p)
+        assert len(out) == 8
+        for t in out:
+            lg = so.forward(cfg, tensors, seq)[-1]
+            third = np.sort(lg)[-3]
+            assert lg[int(t)] >= third - 1e-3, (len(p), len(seq))
+            seq.append(int(t))
+
+
 def test_synthetic_weights_and_state_plan():
     from vllm_rs_amd.engine import Engine
     cfg = checkpoint.parse_config(config_a())

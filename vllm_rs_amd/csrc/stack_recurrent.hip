@@ -152,26 +152,46 @@ __global__ __launch_bounds__(256) void stk_sandwich_kernel(StkSandwichArgs a) {
   if (!a.router_w) return;
   __syncthreads();
   const T* rw = (const T*)a.router_w;
-  for (int e = wave; e < a.n_router; e += 4) {
-    float z = 0.f;
-    if (sizeof(T) == 2 && W % 8 == 0 && ((uintptr_t)rw % 16) == 0) {  // 8 weights a load; a lane's partial sums keep one order for a given W
+  // a wave takes EB outputs at a time and requests their weights together: the rows of one output after the other would each wait for
+  // their own trip to memory.  An output's sum keeps its order (a lane's columns ascending, then the lanes).
+  constexpr int EB = 8;
+  const bool vec8 = sizeof(T) == 2 && W % 8 == 0 && ((uintptr_t)rw % 16) == 0;  // 8 weights a load
+  for (int e0 = wave * EB; e0 < a.n_router; e0 += 4 * EB) {
+    float z[EB];
+#pragma unroll
+    for (int u = 0; u < EB; u++) z[u] = 0.f;
+    if (vec8) {
       for (int c = lane * 8; c < W; c += 64 * 8) {
-        const u32x4 v = *(const u32x4*)((const uint16_t*)rw + (size_t)e * W + c);
-        for (int i = 0; i < 4; i++) {
-          z = fmaf(xs[c + 2 * i], __uint_as_float(v[i] << 16), z);
-          z = fmaf(xs[c + 2 * i + 1], __uint_as_float(v[i] & 0xffff0000u), z);
-        }
+        u32x4 v[EB];
+#pragma unroll
+        for (int u = 0; u < EB; u++) v[u] = *(const u32x4*)((const uint16_t*)rw + (size_t)min(e0 + u, a.n_router - 1) * W + c);
+#pragma unroll
+        for (int u = 0; u < EB; u++)
+          for (int i = 0; i < 4; i++) {
+            z[u] = fmaf(xs[c + 2 * i], __uint_as_float(v[u][i] << 16), z[u]);
+            z[u] = fmaf(xs[c + 2 * i + 1], __uint_as_float(v[u][i] & 0xffff0000u), z[u]);
+          }
       }
     } else {
-      for (int c = lane; c < W; c += 64) z = fmaf(xs[c], El<T>::ld(rw + (size_t)e * W + c), z);
+      for (int c = lane; c < W; c += 64) {
+        float wv[EB];
+#pragma unroll
+        for (int u = 0; u < EB; u++) wv[u] = El<T>::ld(rw + (size_t)min(e0 + u, a.n_router - 1) * W + c);
+#pragma unroll
+        for (int u = 0; u < EB; u++) z[u] = fmaf(xs[c], wv[u], z[u]);
+      }
     }
-    z = wave_sum(z);
-    if (lane == 0) zs[e] = z + (a.router_kind == 0 && a.router_bias ? a.router_bias[e] : 0.f);
+#pragma unroll
+    for (int u = 0; u < EB; u++) {
+      const float zu = wave_sum(z[u]);
+      const int e = e0 + u;
+      if (lane == 0 && e < a.n_router) zs[e] = zu + (a.router_kind == 0 && a.router_bias ? a.router_bias[e] : 0.f);
+    }
   }
   __syncthreads();
-  if (tid != 0) return;
   const int n = a.n_router;
   if (a.router_kind == 0) {  // the `top` largest in turn (ties: the lower index); a picked logit leaves the list
+    if (tid != 0) return;
     float zmax = 0.f, sum = 0.f;
     for (int j = 0; j < a.top; j++) {
       int best = 0;
@@ -189,30 +209,69 @@ __global__ __launch_bounds__(256) void stk_sandwich_kernel(StkSandwichArgs a) {
     for (int j = 0; j < a.top; j++) a.pair_weight[(size_t)t * a.top + j] *= inv;
     return;
   }
-  // scores over all outputs; corrected scores choose, restricted to the best groups; the plain scores weigh
+  // Scores over all outputs; corrected scores choose, restricted to the best groups; the plain scores weigh.  The outputs are spread
+  // over the lanes of wave 0 (their corrections are fetched side by side, not one after the other), the groups over the threads.
   float* sc = zs + n;        // [n] scores
   float* gs = zs + 2 * n;    // [n_groups]
-  float zmax = zs[0], sum = 0.f;
-  for (int e = 1; e < n; e++) zmax = fmaxf(zmax, zs[e]);
-  for (int e = 0; e < n; e++) sc[e] = expf(zs[e] - zmax), sum += sc[e];
-  const float inv = 1.f / sum;
-  for (int e = 0; e < n; e++) sc[e] *= inv, zs[e] = sc[e] + (a.router_bias ? a.router_bias[e] : 0.f);
-  if (a.n_groups > 1 && a.keep < a.n_groups) {
+  if (wave == 0) {
+    float m = -INFINITY, sum = 0.f;
+    for (int e = lane; e < n; e += 64) m = fmaxf(m, zs[e]);
+    m = wave_max(m);
+    for (int e = lane; e < n; e += 64) {
+      const float ex = expf(zs[e] - m);
+      sc[e] = ex;
+      sum += ex;
+    }
+    const float inv = 1.f / wave_sum(sum);
+    for (int e = lane; e < n; e += 64) {
+      const float sv = sc[e] * inv;
+      sc[e] = sv;
+      zs[e] = sv + (a.router_bias ? a.router_bias[e] : 0.f);
+    }
+  }
+  __syncthreads();
+  if (a.n_groups > 1 && a.keep < a.n_groups) {  // (uniform over the workgroup)
     const int per = n / a.n_groups;
-    for (int g = 0; g < a.n_groups; g++) {
+    for (int g = tid; g < a.n_groups; g += 256) {
       float b = zs[g * per];
       for (int e = 1; e < per; e++) b = fmaxf(b, zs[g * per + e]);
       gs[g] = b;
     }
-    for (int g = 0; g < a.n_groups; g++) {  // a group stays if fewer than `keep` groups come before it (larger score, or equal and lower index)
+    __syncthreads();
+    for (int g = tid; g < a.n_groups; g += 256) {  // a group stays if fewer than `keep` groups come before it (larger score, or equal and lower index)
       int before = 0;
       for (int o = 0; o < a.n_groups; o++) before += (gs[o] > gs[g] || (gs[o] == gs[g] && o < g)) ? 1 : 0;
       if (before >= a.keep)
         for (int e = 0; e < per; e++) zs[g * per + e] = -INFINITY;
     }
+    __syncthreads();
   }
-  float idw = 0.f;
   const int n_real = n - a.n_identity;
+  if (n <= 64) {  // one output a lane: a pick is a wave maximum and the lowest lane that holds it
+    if (wave != 0) return;
+    const bool have = lane < n;
+    const float val = have ? zs[lane] : 0.f, sv = have ? sc[lane] : 0.f;
+    bool avail = have;
+    float idw = 0.f;
+    for (int j = 0; j < a.top; j++) {
+      const float v = avail ? val : -INFINITY;
+      const float m = wave_max(v);
+      const unsigned long long holders = __ballot(avail && v == m);  // (left-out groups hold -inf: still chosen, in index order, once nothing else is left)
+      const int best = __ffsll((long long)holders) - 1;
+      const float w = __shfl(sv, best, 64);
+      if (lane == best) avail = false;
+      const bool ident = best >= n_real;
+      if (lane == 0) {
+        a.pair_expert[(size_t)t * a.top + j] = ident ? -1 : best;
+        a.pair_weight[(size_t)t * a.top + j] = w;
+      }
+      if (ident) idw += w;
+    }
+    if (lane == 0 && a.id_weight) a.id_weight[t] = idw;
+    return;
+  }
+  if (tid != 0) return;
+  float idw = 0.f;
   for (int j = 0; j < a.top; j++) {
     int best = -1;
     float bz = -INFINITY;
