@@ -598,7 +598,6 @@ def test_linear_recurrence_forms(form, H, rep, D, V):
     v = r.standard_normal((T, H, V)).astype(np.float32)
     q64, k64, v64 = q.astype(np.float64), k.astype(np.float64), v.astype(np.float64)
     if form == "silu-constant-decay":
-        assert rep == 1 or True
         head_decay = (0.8 + 0.19 * r.random(H)).astype(np.float32)
         ref = so.constant_decay_recurrence(np.repeat(so.silu(q64), rep, 1) * 0.5, np.repeat(so.silu(k64), rep, 1), so.silu(v64), head_decay.astype(np.float64))
         args = dict(decay=None, head_decay=head_decay, beta=None, act=1)

@@ -3,7 +3,8 @@
 //
 //   block   parallel:    x <- x + m * (mixer(h) + ff(h)),  h = norm(x)                      (Ditilix)
 //           sequential:  x <- x + mixer(norm1(x)),  x <- x + ff(norm2(x))                   (Gaperax)
-//           sandwich:    x <- x + norm1b(mixer(norm1(x))),  x <- x + norm2b(ff(norm2(x)))   (Zifetar; RMS norms, norm_offset added to the weights)
+//           sandwich:    x <- x + norm1b(mixer(norm1(x))),  x <- x + norm2b(ff(norm2(x)))   (Zifetar: RMS norms, norm_offset added to the weights;
+//                        Sudosun: Dynamic Tanh norms, the head is the embedding table)
 //   norm    rms: RMS norm over `groups` equal parts of the width;  dyt: Dynamic Tanh  tanh(alpha x) w + b  (no statistics)
 //   pos     sinusoid: a position vector added to the embedding;  none: positions enter inside the mixers
 //   embedding (sandwich stacks): embed * embed_scale + a row of a hashed (previous token, token) table (pair_buckets, pair_mul_prev,
