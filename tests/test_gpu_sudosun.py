@@ -681,7 +681,7 @@ def test_convolution_and_gated_recurrence(dt, C, blocks, taps):
 
 
 @pytest.mark.parametrize("dt", [F32, BF16], ids=["f32", "bf16"])
-@pytest.mark.parametrize("W,E,ident,top,groups,keep", [(96, 6, 3, 3, 3, 2), (51, 3, 0, 3, 0, 0), (256, 36, 4, 1, 8, 3), (64, 6, 2, 4, 4, 1)])
+@pytest.mark.parametrize("W,E,ident,top,groups,keep", [(96, 6, 3, 3, 3, 2), (51, 3, 0, 3, 0, 0), (256, 36, 4, 1, 8, 3), (64, 6, 2, 4, 4, 1), (128, 70, 2, 3, 8, 3)])
 def test_seam_with_dynamic_tanh_and_grouped_router(dt, W, E, ident, top, groups, keep):
     """x += D(c1 N(part1) + c2 N(part2); post), h = D(x; pre) with D = tanh(alpha v) w + b and N an RMS norm of the part's own; then pairs
     without a row and a weighted second part; the router: softmax over all outputs, choice by corrected score inside the best groups,
